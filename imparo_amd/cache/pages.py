@@ -113,9 +113,12 @@ class PagedSpec:
     per position (keys and values, a latent, whatever it declares), laid out
     as the mixer's kernels read them. `window` None keeps every position; a
     number keeps only that many. Sites with equal specs share a pool and a
-    block table per request."""
+    block table per request. `fixed`: what the site keeps per request beside
+    its pages, of a fixed size (the input its last token left, for a layer that
+    mixes every token with the one before it)."""
     arrays: Tuple[PagedArray, ...]
     window: Optional[int] = None
+    fixed: Optional["FixedSpec"] = None
 
     def __post_init__(self):
         names = [a.name for a in self.arrays]
@@ -176,6 +179,27 @@ class FixedSpec:
 
 
 StateSpec = Union[PagedSpec, FixedSpec, None]
+
+
+def fixed_part(spec: StateSpec) -> Optional[FixedSpec]:
+    """What a site keeps per request in a state slot: a fixed spec itself, or a paged spec's `fixed`."""
+    if isinstance(spec, FixedSpec):
+        return spec
+    if isinstance(spec, PagedSpec):
+        return spec.fixed
+    return None
+
+
+def with_fixed_arrays(spec: StateSpec, arrays: Sequence[FixedArray]) -> StateSpec:
+    """`spec` with further fixed-size arrays per request: what a block adds to its mixer's state."""
+    arrays = tuple(arrays)
+    if not arrays:
+        return spec
+    old = fixed_part(spec)
+    both = FixedSpec(arrays=(old.all_arrays() if old is not None else ()) + arrays)
+    if isinstance(spec, PagedSpec):
+        return PagedSpec(spec.arrays, spec.window, both)
+    return both
 
 
 class _Tables:
@@ -299,7 +323,7 @@ class CacheManager:
             grp = CacheGroup(self, g, spec, pool, page_size)
             grp.sites = sites_of[g]
             self.groups.append(grp)
-        self.fixed_sites = [s for s, spec in enumerate(self.site_specs) if isinstance(spec, FixedSpec)]
+        self.fixed_sites = [s for s, spec in enumerate(self.site_specs) if fixed_part(spec) is not None]
         self.n_slots = n_slots
         self.slots = PagePool(0, _borrowed=self._lib.imparo_cache_slot_pool(self._c))
         self._handles: Dict[Hashable, int] = {}

@@ -1,5 +1,8 @@
 """The device memory behind the cache manager's pages and slots.
 
+A site with a paged spec that also names fixed-size state (`PagedSpec.fixed`)
+gets both.
+
 Per cache site with a paged spec: one tensor per array the spec declares,
 [n_pages of the site's group, *the array's page shape], in the engine's dtype
 or in float32 as the array says. The layout inside a page is the mixer's
@@ -14,7 +17,7 @@ from typing import Dict, Tuple
 import torch
 
 from ..kernels import ops
-from .pages import CacheManager, FixedSpec, PagedSpec
+from .pages import CacheManager, PagedSpec, fixed_part
 
 
 class CacheStorage:
@@ -32,10 +35,11 @@ class CacheStorage:
                     a.name: torch.zeros(a.shape(n_pages, manager.page_size),
                                         dtype=torch.float32 if a.float32 else dtype, device=device)
                     for a in spec.arrays}
-            elif isinstance(spec, FixedSpec):
+            fixed = fixed_part(spec)
+            if fixed is not None:
                 kinds = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32, "engine": dtype}
                 arrays = {a.name: torch.full((manager.n_slots,) + tuple(a.shape), a.init, dtype=kinds[a.dtype],
-                                             device=device) for a in spec.all_arrays()}
+                                             device=device) for a in fixed.all_arrays()}
                 self.fixed_arrays[site] = arrays
                 if len(arrays) == 1 or "state" in arrays:
                     self.fixed[site] = arrays.get("state", next(iter(arrays.values())))
@@ -44,7 +48,7 @@ class CacheStorage:
         # dtype) and takes a whole number of words per slot.
         resets = []
         for site in sorted(self.fixed_arrays):
-            for a in manager.site_specs[site].all_arrays():
+            for a in fixed_part(manager.site_specs[site]).all_arrays():
                 t = self.fixed_arrays[site][a.name]
                 per_slot = t[0].numel() * t.element_size()
                 if per_slot % 4:

@@ -6,3 +6,7 @@ from . import lfm2 as _lfm2
 from .lfm2 import Lfm2Config, adjusted_ff_dim
 
 register_architecture(_lfm2.ARCHITECTURE, Lfm2Config.from_dict, _lfm2.build_plan)
+from . import tumadra as _tumadra
+from .tumadra import TumadraConfig
+
+register_architecture(_tumadra.ARCHITECTURE, TumadraConfig.from_dict, _tumadra.build_plan)

@@ -2,7 +2,8 @@
 
 The reference keys the same table by the file's architecture string
 (/root/reference/crates/imparo-model/src/lib.rs:2958-2970). Here the key is
-config.json's `architectures[0]`.
+config.json's `architectures[0]`, or its `architecture` where a file names
+its one architecture as a string.
 """
 from __future__ import annotations
 
@@ -36,8 +37,10 @@ def known_architectures() -> Tuple[str, ...]:
 
 def architecture_of(config: Dict[str, Any]) -> Architecture:
     archs = config.get("architectures")
+    if archs is None and isinstance(config.get("architecture"), str):
+        archs = [config["architecture"]]
     if archs is None:
-        raise MissingKey("config.json: required key 'architectures' is missing")
+        raise MissingKey("config.json: required key 'architectures' (or 'architecture') is missing")
     if not isinstance(archs, list) or len(archs) == 0 or not isinstance(archs[0], str):
         raise BadValue("config.json: architectures must be a non-empty list of names")
     name = archs[0]

@@ -216,6 +216,61 @@ int imparo_fill_f32(float* p, float value, int64_t n, imparo_stream stream);
 int imparo_fill_sites(const uint64_t* base, const int64_t* per_slot, const float* value, int n_sites, int slot,
                       imparo_stream stream);
 
+// ---- row-wise kernels of layers that norm in groups, shift tokens, add a sinusoid or use a polynomial activation
+// x[t, 2i] = table[ids[t], 2i] + sin(positions[t] * inv_freq[i]), x[t, 2i + 1] = ... + cos(the same angle).
+int imparo_embed_sinusoid(const void* table, int table_dtype, const int32_t* ids, const int32_t* positions,
+                          const float* inv_freq, float* x, int n_tokens, int width, int vocab, imparo_stream stream);
+// imparo_rms_norm with the row cut into `groups` equal consecutive parts, each divided by its own root mean
+// square. With shift_mix [width] (rows of one token each, row i's request in slot[i]; rows must be null):
+// out = h + (prev - h) * mix with prev = shift_state[slot[i]], which then becomes h (float32 [slots, width]).
+int imparo_group_rms_norm(float* x, const float* delta, int n_delta, int n_x_rows, const int32_t* rows,
+                          const float* weight, void* out, int out_dtype, int n_rows, int width, int groups, float eps,
+                          int write_back, const float* shift_mix, float* shift_state, const int32_t* slot,
+                          imparo_stream stream);
+// out[t] = h[t] + (prev - h[t]) * mix, prev the row before inside a request's segment and state[slot] at its
+// first token; afterwards state[slot] = the segment's last row of h. h float32 [tokens, width].
+int imparo_token_shift(const float* h, const float* mix, float* state, const int32_t* row_of_token,
+                       const int32_t* seg_start, const int32_t* seg_len, const int32_t* slot, void* out, int out_dtype,
+                       int n_tokens, int n_rows, int width, imparo_stream stream);
+// out = a N(z) + b N(z^2) + c N(z^3) + e with N(v) = v / sqrt(mean(v^2) + eps) over a token's `width` values;
+// coef = {a, b, c, e} on the device. Columns width .. out_ld of out become zero.
+int imparo_poly_norm(const float* z, int z_ld, const float* coef, void* out, int out_dtype, int out_ld, int n_tokens,
+                     int width, float eps, imparo_stream stream);
+
+// ---- selective state-space mixer
+// y[t, c] = act(bias[c] + sum_k weight[c, k] u[t - (taps - 1) + k, c]) per request, zeros before its start;
+// state [slots, taps - 1, channels] float32 holds each request's last inputs and is advanced. u rows lie u_ld
+// floats apart. single_tokens: every row brings one token (one launch instead of two).
+int imparo_causal_conv(const float* u, int u_ld, const float* weight, const float* bias, float* state,
+                       const int32_t* row_of_token, const int32_t* seg_start, const int32_t* seg_len,
+                       const int32_t* slot, void* out, int out_dtype, int n_tokens, int n_rows, int channels, int taps,
+                       int silu, int single_tokens, imparo_stream stream);
+// S[c, n] <- exp(dt A[c, n]) S[c, n] + dt x[c] B[n]; y[c] = sum_n S[c, n] C[n] + D[c] x[c]; out = y * silu(z);
+// dt = softplus(dt_raw). bc rows are [B | C] float32; state [slots, channels, n_state] float32.
+int imparo_selective_scan(const float* dt_raw, const void* x, const float* bc, const float* z, int z_ld,
+                          const float* A, const float* D, float* state, const int32_t* seg_start,
+                          const int32_t* seg_len, const int32_t* slot, void* out, int dtype, int n_rows, int channels,
+                          int n_state, imparo_stream stream);
+
+// ---- differential attention (two softmax maps a head over shared values)
+// rows_in float32 [tokens, ld] = [q: heads x 2 x dim | k: kv_heads x 2 x dim | v: kv_heads x vdim | ...];
+// q_out [tokens, heads, 2, dim] = q * (1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)) (temp_every 0:
+// none); with write_kv, k and v go into their pages: K [n_pages, 2 kv_heads, page_size, dim], V [n_pages,
+// kv_heads, page_size, vdim].
+int imparo_diff_qkv_store(const float* rows_in, int ld, const int32_t* positions, const int32_t* row_of_token,
+                          const int32_t* block_table, int table_stride, int page_size, void* q_out, void* k_cache,
+                          void* v_cache, int dtype, int write_kv, int n_tokens, int heads, int kv_heads, int dim,
+                          int vdim, int n_pages, float temp_coef, int temp_every, imparo_stream stream);
+// Per (token, head): a_m = softmax_j(q_m . k_m[j] * scale) v[j] over the keys lo..pos, o = a_1 - lambda a_2,
+// out = o / sqrt(mean(o^2) + eps) * out_scale * sigmoid(gate) (gate null: no gate). n_splits > 1 walks the
+// keys in pieces of imparo_diff_attention_split() through `part` (tokens x heads x n_splits x (2 vdim + 4) floats).
+int imparo_diff_attention_split(void);
+int imparo_diff_attention(const void* q, const void* k_cache, const void* v_cache, const float* gate, int gate_ld,
+                          void* out, float* part, int dtype, const int32_t* positions, const int32_t* row_of_token,
+                          const int32_t* block_table, int table_stride, int page_size, int n_tokens, int heads,
+                          int kv_heads, int dim, int vdim, int n_pages, float scale, int window, float lambda,
+                          float eps, float out_scale, int n_splits, imparo_stream stream);
+
 // ---------------------------------------------------------------------------------------------
 // A model's step as one call. A program is the model's run order as a list of operations over a
 // float32 residual stream: the embedding, then per layer a norm, a mixer, a norm and a

@@ -117,10 +117,13 @@ __device__ __forceinline__ void wave_lds_sync() {
 int imparo_load_code_attention();
 int imparo_load_code_attention_mfma();
 int imparo_load_code_decode_rows();
+int imparo_load_code_diff_attention();
 int imparo_load_code_elementwise();
 int imparo_load_code_gemm();
 int imparo_load_code_rope_cache();
+int imparo_load_code_row_ops();
 int imparo_load_code_sampling();
+int imparo_load_code_selective_scan();
 
 static inline int launch_status() {
     return hipGetLastError() == hipSuccess ? IMPARO_OK : IMPARO_LAUNCH_FAILED;

@@ -1,0 +1,367 @@
+// Differential attention over the paged cache: every head holds two softmax maps over the same
+// values, combined as a1 - lambda a2, brought to unit RMS per head, scaled, gated and stored.
+//
+// Cache layout: K [n_pages, 2 kv_heads, page_size, dim] (key head g's map m is row 2g + m), V
+// [n_pages, kv_heads, page_size, vdim]. Queries [tokens, heads, 2, dim] arrive already multiplied by
+// their position's temperature. Scores, softmax, the combination and the norm are float32.
+//
+// k_diff_qkv_store: from the fused projection's float32 rows [q | k | v | ...] the queries (times the
+// temperature 1 + coef * ln(floor((pos + 1) / every) + 1)) and the new keys and values into their pages.
+// k_diff_attention: one wave per (token, head, split of the keys). Keys are walked in chunks of 64 at
+// absolute multiples of 64, one key a lane for the two scores, one value dimension a lane for the two
+// weighted sums; both maps share every value load. With one split the wave finishes the head itself;
+// with more, the splits (DA_SPLIT keys each, at absolute multiples) leave their running maxima, sums
+// and weighted sums, and k_diff_merge finishes.
+#include "common.h"
+#include "api.h"
+
+#define DA_WAVES 4
+#define DA_MAX_DIM 256
+#define DA_MAX_VDIM 512
+#define DA_DPL (DA_MAX_VDIM / WAVE)
+#define DA_SPLIT 256
+
+extern "C" int imparo_diff_attention_split(void) { return DA_SPLIT; }
+
+template <typename T>
+__global__ void k_diff_qkv_store(const float* __restrict__ rows_in, int ld, const int32_t* __restrict__ positions,
+                                 const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ block_table,
+                                 int table_stride, int page_size, T* __restrict__ q_out, T* __restrict__ k_cache,
+                                 T* __restrict__ v_cache, int write_kv, int heads, int kv_heads, int dim, int vdim,
+                                 int n_pages, float temp_coef, int temp_every) {
+    const int t = blockIdx.x;
+    const int pos = positions[t];
+    const float* row = rows_in + (size_t)t * ld;
+    const int nq = heads * 2 * dim, nk = kv_heads * 2 * dim, nv = kv_heads * vdim;
+    float temp = 1.0f;
+    if (temp_every > 0) temp = 1.0f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.0f);
+    for (int i = threadIdx.x; i < nq; i += blockDim.x) store_f32<T>(q_out, (size_t)t * nq + i, row[i] * temp);
+    if (!write_kv) return;
+    const int page = block_table[(size_t)row_of_token[t] * table_stride + pos / page_size];
+    if (page < 0 || page >= n_pages) return;
+    const int in_page = pos % page_size;
+    for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+        const int kh = i / dim, d = i - kh * dim;
+        store_f32<T>(k_cache, (((size_t)page * 2 * kv_heads + kh) * page_size + in_page) * dim + d, row[nq + i]);
+    }
+    for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+        const int g = i / vdim, d = i - g * vdim;
+        store_f32<T>(v_cache, (((size_t)page * kv_heads + g) * page_size + in_page) * vdim + d, row[nq + nk + i]);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ float da_dot(const float* __restrict__ q, const T* __restrict__ k, int dim);
+
+// 16 bytes a load where the rows allow it (every key row then starts at a multiple of 16 bytes)
+template <>
+__device__ __forceinline__ float da_dot<float>(const float* __restrict__ q, const float* __restrict__ k, int dim) {
+    float s = 0.f;
+    if ((dim & 3) == 0) {
+        for (int i = 0; i < dim; i += 4) {
+            const float4 kv = *reinterpret_cast<const float4*>(k + i);
+            s += q[i] * kv.x;
+            s += q[i + 1] * kv.y;
+            s += q[i + 2] * kv.z;
+            s += q[i + 3] * kv.w;
+        }
+    } else {
+        for (int i = 0; i < dim; ++i) s += q[i] * k[i];
+    }
+    return s;
+}
+
+template <>
+__device__ __forceinline__ float da_dot<bf16_t>(const float* __restrict__ q, const bf16_t* __restrict__ k, int dim) {
+    float s = 0.f;
+    if ((dim & 7) == 0) {
+        for (int i = 0; i < dim; i += 8) {
+            const uint4 kv = *reinterpret_cast<const uint4*>(k + i);
+            const uint32_t w[4] = {kv.x, kv.y, kv.z, kv.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                s += q[i + 2 * j] * __uint_as_float(w[j] << 16);
+                s += q[i + 2 * j + 1] * __uint_as_float(w[j] & 0xffff0000u);
+            }
+        }
+    } else {
+        for (int i = 0; i < dim; ++i) s += q[i] * bf16_to_f32(k[i]);
+    }
+    return s;
+}
+
+// What finishes a head: o = a1 - lambda a2 over the head's vdim values (lane d holds d, d + 64, ...), divided
+// by its root mean square, times out_scale, times sigmoid(gate).
+template <typename T>
+__device__ __forceinline__ void da_finish(const float (&a1)[DA_DPL], const float (&a2)[DA_DPL], float lambda, float eps,
+                                          float out_scale, const float* __restrict__ gate, T* __restrict__ dst, int vdim,
+                                          int lane) {
+    float o[DA_DPL];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < DA_DPL; ++j) {
+        const int d = lane + j * WAVE;
+        o[j] = d < vdim ? a1[j] - lambda * a2[j] : 0.f;
+        ss += o[j] * o[j];
+    }
+    ss = wave_sum(ss);
+    const float r = out_scale / sqrtf(ss / (float)vdim + eps);
+#pragma unroll
+    for (int j = 0; j < DA_DPL; ++j) {
+        const int d = lane + j * WAVE;
+        if (d < vdim) {
+            float y = o[j] * r;
+            if (gate) y *= 1.0f / (1.0f + expf(-gate[d]));
+            store_f32<T>(dst, d, y);
+        }
+    }
+}
+
+template <typename T>
+__global__ void k_diff_attention(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                                 const float* __restrict__ gate, int gate_ld, T* __restrict__ out,
+                                 float* __restrict__ part, const int32_t* __restrict__ positions,
+                                 const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ block_table,
+                                 int table_stride, int page_size, int n_tokens, int heads, int kv_heads, int dim,
+                                 int vdim, int n_pages, float scale, int window, float lambda, float eps,
+                                 float out_scale, int n_splits) {
+    __shared__ float q_rows[DA_WAVES][2 * DA_MAX_DIM];
+    __shared__ float probs[DA_WAVES][2][WAVE];
+    __shared__ long long v_off[DA_WAVES][WAVE];
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x / WAVE;
+    const long long id = (long long)blockIdx.x * DA_WAVES + wave;
+    if (id >= (long long)n_tokens * heads * n_splits) return;
+    const int split = (int)(id % n_splits);
+    const long long th = id / n_splits;
+    const int t = (int)(th / heads);
+    const int h = (int)(th - (long long)t * heads);
+    const int g = h / (heads / kv_heads);
+    const int pos = positions[t];
+    const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    int first = (lo / WAVE) * WAVE, last = pos;             // chunks from `first`, keys up to `last`
+    if (n_splits > 1) {
+        first = max(first, split * DA_SPLIT);
+        last = min(pos, (split + 1) * DA_SPLIT - 1);
+        if (first > last) return;                             // this split holds no key of the query (uniform over the wave)
+    }
+    const int32_t* table = block_table + (size_t)row_of_token[t] * table_stride;
+
+    float* qr = q_rows[wave];
+    const T* qsrc = q + ((size_t)t * heads + h) * 2 * dim;
+    for (int i = lane; i < 2 * dim; i += WAVE) qr[i] = load_f32<T>(qsrc, i);
+    wave_lds_sync();
+
+    float a1[DA_DPL], a2[DA_DPL];
+#pragma unroll
+    for (int j = 0; j < DA_DPL; ++j) a1[j] = a2[j] = 0.f;
+    float m1 = -INFINITY, l1 = 0.f, m2 = -INFINITY, l2 = 0.f;
+
+    for (int c = first; c <= last; c += WAVE) {
+        const int p = c + lane;
+        const bool valid = p >= lo && p <= last;
+        float s1 = -INFINITY, s2 = -INFINITY;
+        long long off = -1;
+        if (valid) {
+            const int page = table[p / page_size];
+            if (page >= 0 && page < n_pages) {
+                const long long k_off = (((long long)page * 2 * kv_heads + 2 * g) * page_size + (p % page_size)) * dim;
+                s1 = da_dot<T>(qr, k_cache + k_off, dim) * scale;
+                s2 = da_dot<T>(qr + dim, k_cache + k_off + (long long)page_size * dim, dim) * scale;
+                off = (((long long)page * kv_heads + g) * page_size + (p % page_size)) * vdim;
+            }
+        }
+        const float m1n = fmaxf(m1, wave_max(s1));
+        const float m2n = fmaxf(m2, wave_max(s2));
+        const float p1 = off >= 0 ? expf(s1 - m1n) : 0.f;
+        const float p2 = off >= 0 ? expf(s2 - m2n) : 0.f;
+        const float c1 = m1 == -INFINITY ? 0.f : expf(m1 - m1n);
+        const float c2 = m2 == -INFINITY ? 0.f : expf(m2 - m2n);
+        l1 = l1 * c1 + wave_sum(p1);
+        l2 = l2 * c2 + wave_sum(p2);
+        m1 = m1n;
+        m2 = m2n;
+        probs[wave][0][lane] = p1;
+        probs[wave][1][lane] = p2;
+        v_off[wave][lane] = off;
+        wave_lds_sync();
+        const int n_keys = min(WAVE, last - c + 1);
+#pragma unroll
+        for (int j = 0; j < DA_DPL; ++j) {
+            a1[j] *= c1;
+            a2[j] *= c2;
+        }
+        for (int kk = 0; kk < n_keys; ++kk) {
+            const long long vo = v_off[wave][kk];
+            if (vo < 0) continue;                 // uniform over the wave
+            const float w1 = probs[wave][0][kk], w2 = probs[wave][1][kk];
+            const T* vrow = v_cache + vo;
+#pragma unroll
+            for (int j = 0; j < DA_DPL; ++j) {
+                const int d = lane + j * WAVE;
+                if (d < vdim) {
+                    const float v = load_f32<T>(vrow, d);
+                    a1[j] += w1 * v;
+                    a2[j] += w2 * v;
+                }
+            }
+        }
+        wave_lds_sync();
+    }
+    if (n_splits > 1) {
+        float* dst = part + ((size_t)th * n_splits + split) * (2 * vdim + 4);
+        if (lane == 0) {
+            dst[0] = m1;
+            dst[1] = l1;
+            dst[2] = m2;
+            dst[3] = l2;
+        }
+#pragma unroll
+        for (int j = 0; j < DA_DPL; ++j) {
+            const int d = lane + j * WAVE;
+            if (d < vdim) {
+                dst[4 + d] = a1[j];
+                dst[4 + vdim + d] = a2[j];
+            }
+        }
+        return;
+    }
+    const float i1 = l1 > 0.f ? 1.0f / l1 : 0.f, i2 = l2 > 0.f ? 1.0f / l2 : 0.f;
+#pragma unroll
+    for (int j = 0; j < DA_DPL; ++j) {
+        a1[j] *= i1;
+        a2[j] *= i2;
+    }
+    da_finish<T>(a1, a2, lambda, eps, out_scale, gate ? gate + (size_t)t * gate_ld + (size_t)h * vdim : nullptr,
+                 out + ((size_t)t * heads + h) * vdim, vdim, lane);
+}
+
+// One wave per (token, head): the splits that hold keys of the query, in order.
+template <typename T>
+__global__ void k_diff_merge(const float* __restrict__ part, const float* __restrict__ gate, int gate_ld,
+                             T* __restrict__ out, const int32_t* __restrict__ positions, int n_tokens, int heads,
+                             int vdim, int window, float lambda, float eps, float out_scale, int n_splits) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const long long th = (long long)blockIdx.x * DA_WAVES + threadIdx.x / WAVE;
+    if (th >= (long long)n_tokens * heads) return;
+    const int t = (int)(th / heads);
+    const int h = (int)(th - (long long)t * heads);
+    const int pos = positions[t];
+    const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    const int s_first = lo / DA_SPLIT, s_last = min(pos / DA_SPLIT, n_splits - 1);
+    const float* base = part + (size_t)th * n_splits * (2 * vdim + 4);
+    float m1 = -INFINITY, m2 = -INFINITY;
+    for (int s = s_first; s <= s_last; ++s) {
+        const float* p = base + (size_t)s * (2 * vdim + 4);
+        m1 = fmaxf(m1, p[0]);
+        m2 = fmaxf(m2, p[2]);
+    }
+    float a1[DA_DPL], a2[DA_DPL];
+#pragma unroll
+    for (int j = 0; j < DA_DPL; ++j) a1[j] = a2[j] = 0.f;
+    float l1 = 0.f, l2 = 0.f;
+    for (int s = s_first; s <= s_last; ++s) {
+        const float* p = base + (size_t)s * (2 * vdim + 4);
+        const float w1 = p[0] == -INFINITY ? 0.f : expf(p[0] - m1);
+        const float w2 = p[2] == -INFINITY ? 0.f : expf(p[2] - m2);
+        l1 += w1 * p[1];
+        l2 += w2 * p[3];
+#pragma unroll
+        for (int j = 0; j < DA_DPL; ++j) {
+            const int d = lane + j * WAVE;
+            if (d < vdim) {
+                a1[j] += w1 * p[4 + d];
+                a2[j] += w2 * p[4 + vdim + d];
+            }
+        }
+    }
+    const float i1 = l1 > 0.f ? 1.0f / l1 : 0.f, i2 = l2 > 0.f ? 1.0f / l2 : 0.f;
+#pragma unroll
+    for (int j = 0; j < DA_DPL; ++j) {
+        a1[j] *= i1;
+        a2[j] *= i2;
+    }
+    da_finish<T>(a1, a2, lambda, eps, out_scale, gate ? gate + (size_t)t * gate_ld + (size_t)h * vdim : nullptr,
+                 out + ((size_t)t * heads + h) * vdim, vdim, lane);
+}
+
+extern "C" int imparo_diff_qkv_store(const float* rows_in, int ld, const int32_t* positions, const int32_t* row_of_token,
+                                     const int32_t* block_table, int table_stride, int page_size, void* q_out,
+                                     void* k_cache, void* v_cache, int dtype, int write_kv, int n_tokens, int heads,
+                                     int kv_heads, int dim, int vdim, int n_pages, float temp_coef, int temp_every,
+                                     imparo_stream stream) {
+    if (!rows_in || !positions || !row_of_token || !q_out) return IMPARO_BAD_ARGUMENT;
+    if (write_kv && (!block_table || !k_cache || !v_cache || table_stride <= 0 || n_pages <= 0)) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0 || page_size <= 0)
+        return IMPARO_BAD_ARGUMENT;
+    if (ld < (heads + kv_heads) * 2 * dim + kv_heads * vdim || temp_every < 0) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == IMPARO_F32)
+        k_diff_qkv_store<float><<<n_tokens, 256, 0, s>>>(rows_in, ld, positions, row_of_token, block_table, table_stride,
+                                                         page_size, (float*)q_out, (float*)k_cache, (float*)v_cache, write_kv,
+                                                         heads, kv_heads, dim, vdim, n_pages, temp_coef, temp_every);
+    else if (dtype == IMPARO_BF16)
+        k_diff_qkv_store<bf16_t><<<n_tokens, 256, 0, s>>>(rows_in, ld, positions, row_of_token, block_table, table_stride,
+                                                          page_size, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                                                          write_kv, heads, kv_heads, dim, vdim, n_pages, temp_coef, temp_every);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
+// q [tokens, heads, 2, dim]; gate (may be null) float32 rows gate_ld apart, heads * vdim values a row, the
+// gate's logits; out [tokens, heads * vdim]. n_splits 1: no partial results; more: part holds
+// tokens * heads * n_splits * (2 vdim + 4) floats and n_splits covers every key (ceil(longest context / split)).
+extern "C" int imparo_diff_attention(const void* q, const void* k_cache, const void* v_cache, const float* gate,
+                                     int gate_ld, void* out, float* part, int dtype, const int32_t* positions,
+                                     const int32_t* row_of_token, const int32_t* block_table, int table_stride,
+                                     int page_size, int n_tokens, int heads, int kv_heads, int dim, int vdim,
+                                     int n_pages, float scale, int window, float lambda, float eps, float out_scale,
+                                     int n_splits, imparo_stream stream) {
+    if (!q || !k_cache || !v_cache || !out || !positions || !row_of_token || !block_table) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads) return IMPARO_BAD_ARGUMENT;
+    if (dim <= 0 || dim > DA_MAX_DIM || vdim <= 0 || vdim > DA_MAX_VDIM) return IMPARO_BAD_ARGUMENT;
+    if (page_size <= 0 || table_stride <= 0 || n_pages <= 0 || window < 0 || n_splits < 1) return IMPARO_BAD_ARGUMENT;
+    if (n_splits > 1 && !part) return IMPARO_BAD_ARGUMENT;
+    if (gate && gate_ld < heads * vdim) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    const long long total = (long long)n_tokens * heads * n_splits;
+    const long long blocks = (total + DA_WAVES - 1) / DA_WAVES;
+    if (blocks > 0x7fffffffLL) return IMPARO_BAD_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    const unsigned merge_blocks = (unsigned)(((long long)n_tokens * heads + DA_WAVES - 1) / DA_WAVES);
+    if (dtype == IMPARO_F32) {
+        k_diff_attention<float><<<(unsigned)blocks, DA_WAVES * WAVE, 0, s>>>(
+            (const float*)q, (const float*)k_cache, (const float*)v_cache, gate, gate_ld, (float*)out, part, positions,
+            row_of_token, block_table, table_stride, page_size, n_tokens, heads, kv_heads, dim, vdim, n_pages, scale,
+            window, lambda, eps, out_scale, n_splits);
+        if (n_splits > 1) {
+            if (launch_status()) return IMPARO_LAUNCH_FAILED;
+            k_diff_merge<float><<<merge_blocks, DA_WAVES * WAVE, 0, s>>>(part, gate, gate_ld, (float*)out, positions,
+                                                                         n_tokens, heads, vdim, window, lambda, eps,
+                                                                         out_scale, n_splits);
+        }
+    } else if (dtype == IMPARO_BF16) {
+        k_diff_attention<bf16_t><<<(unsigned)blocks, DA_WAVES * WAVE, 0, s>>>(
+            (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, gate, gate_ld, (bf16_t*)out, part, positions,
+            row_of_token, block_table, table_stride, page_size, n_tokens, heads, kv_heads, dim, vdim, n_pages, scale,
+            window, lambda, eps, out_scale, n_splits);
+        if (n_splits > 1) {
+            if (launch_status()) return IMPARO_LAUNCH_FAILED;
+            k_diff_merge<bf16_t><<<merge_blocks, DA_WAVES * WAVE, 0, s>>>(part, gate, gate_ld, (bf16_t*)out, positions,
+                                                                          n_tokens, heads, vdim, window, lambda, eps,
+                                                                          out_scale, n_splits);
+        }
+    } else {
+        return IMPARO_BAD_ARGUMENT;
+    }
+    return launch_status();
+}
+
+int imparo_load_code_diff_attention() {
+    hipFuncAttributes attributes;
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_diff_attention<float>)) == hipSuccess
+               ? IMPARO_OK
+               : IMPARO_LAUNCH_FAILED;
+}

@@ -101,7 +101,7 @@ class Model:
             return None
         blocks_emit = all(emits(b) and getattr(b, "can_emit", lambda: True)() for b in self.blocks)
         if not (blocks_emit and emits(self.embedding) and emits(self.final_norm, "emit_head", "forward_rows")
-                and emits(self.head, "emit_projection")):
+                and getattr(self.final_norm, "can_emit", lambda: True)() and emits(self.head, "emit_projection")):
             return None
         program = Program(self.dtype, page_size, storage, group_of_site)
         self.embedding.emit(program)

@@ -50,6 +50,17 @@ _SIGNATURES = {
     "imparo_fill_sites": [P, P, P, I, I, P],
     "imparo_attention_decode_static": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
     "imparo_load_code": [],
+    "imparo_embed_sinusoid": [P, I, P, P, P, P, I, I, I, P],
+    "imparo_group_rms_norm": [P, P, I, I, P, P, P, I, I, I, I, F, I, P, P, P, P],
+    "imparo_token_shift": [P, P, P, P, P, P, P, P, I, I, I, I, P],
+    "imparo_poly_norm": [P, I, P, P, I, I, I, I, F, P],
+    "imparo_causal_conv": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+    "imparo_selective_scan": [P, P, P, P, I, P, P, P, P, P, P, P, I, I, I, I, P],
+    "imparo_diff_qkv_store": [P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
+    "imparo_diff_attention_split": [],
+    # q, k_cache, v_cache, gate, gate_ld, out, part, dtype, positions, row_of_token, table, stride, page, tokens, heads,
+    # kv_heads, dim, vdim, n_pages, scale, window, lambda, eps, out_scale, n_splits, stream
+    "imparo_diff_attention": [P, P, P, P, I, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, F, F, F, I, P],
     "imparo_rows_parts": [I],
     # x, ssq_in, n_parts, eps, w, bias, y, out_dtype, x_io, ssq_out, weighted_out, weighted_by, m, n, k, epilogue, stream
     "imparo_rows_gemm": [P, P, I, F, P, P, P, I, P, P, P, P, I, I, I, I, P],

@@ -506,3 +506,184 @@ def fill_sites(base: torch.Tensor, per_slot: torch.Tensor, value: torch.Tensor, 
                                        _dev(per_slot, "site row sizes", torch.int64, (n,)),
                                        _dev(value, "site values", torch.float32, (n,)), n, int(slot), _stream()),
            "fill_sites")
+
+
+# ------------------------------------------------------------------ grouped norm, token shift, sinusoid, polynomial
+def embed_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
+                   out: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[ids[t]] + the sinusoidal vector of positions[t]: entry 2i is sin(pos * inv_freq[i]),
+    entry 2i + 1 the cosine of the same angle."""
+    vocab, width = table.shape
+    n = ids.shape[0]
+    _check(library().imparo_embed_sinusoid(
+        _dev(table, "embedding table"), _code(table, "embedding table"), _dev(ids, "token ids", torch.int32, (n,)),
+        _dev(positions, "positions", torch.int32, (n,)), _dev(inv_freq, "inverse frequencies", torch.float32, ((width + 1) // 2,)),
+        _dev(out, "embedding output", torch.float32, (n, width)), n, width, vocab, _stream()), "embed_sinusoid")
+    return out
+
+
+def group_rms_norm(x: torch.Tensor, weight: torch.Tensor, groups: int, eps: float, out: torch.Tensor,
+                   delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None, write_back: bool = False,
+                   shift_mix: Optional[torch.Tensor] = None, shift_state: Optional[torch.Tensor] = None,
+                   slot: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`rms_norm` with the row in `groups` equal consecutive parts, each divided by its own root mean square.
+    With `shift_mix` [width], for rows of one token each (row i's request in slot[i]): out = h + (prev - h) *
+    mix, where prev = shift_state[slot[i]] is replaced by h, the normed row."""
+    width = x.shape[-1]
+    n_out = out.shape[0]
+    if groups < 1 or width % groups:
+        raise KernelArgumentError(f"group_rms_norm: {width} values do not make {groups} equal parts")
+    if rows is None and n_out != x.shape[0]:
+        raise KernelArgumentError(f"group_rms_norm: out has {n_out} rows, x has {x.shape[0]}")
+    if rows is not None and rows.shape[0] != n_out:
+        raise KernelArgumentError("group_rms_norm: one source row index per output row is needed")
+    if write_back and (rows is not None or delta is None):
+        raise KernelArgumentError("group_rms_norm: write_back needs a delta and no row selection")
+    n_delta = 0
+    if delta is not None:
+        n_delta = delta.shape[0] if delta.dim() == x.dim() + 1 else 1
+        want = (n_delta,) + tuple(x.shape) if delta.dim() == x.dim() + 1 else tuple(x.shape)
+        _dev(delta, "group_rms_norm delta", torch.float32, want)
+    if shift_mix is not None:
+        if rows is not None or shift_state is None or slot is None or shift_state.dim() != 2:
+            raise KernelArgumentError("group_rms_norm: a token shift needs its state, the rows' slots and no row selection")
+        _dev(shift_state, "shift state", torch.float32, (shift_state.shape[0], width))
+        _dev(slot, "slot", torch.int32, (n_out,))
+    _check(library().imparo_group_rms_norm(
+        _dev(x, "group_rms_norm x", torch.float32), _dev(delta, "group_rms_norm delta", torch.float32), n_delta, x.shape[0],
+        _dev(rows, "group_rms_norm rows", torch.int32), _dev(weight, "group_rms_norm weight", torch.float32, (width,)),
+        _dev(out, "group_rms_norm out", None, (n_out, width)), _code(out, "group_rms_norm out"), n_out, width, int(groups),
+        float(eps), int(write_back), _dev(shift_mix, "shift mix", torch.float32, (width,)),
+        _dev(shift_state, "shift state", torch.float32), _dev(slot, "slot", torch.int32), _stream()), "group_rms_norm")
+    return out
+
+
+def token_shift(h: torch.Tensor, mix: torch.Tensor, state: torch.Tensor, row_of_token: torch.Tensor,
+                seg_start: torch.Tensor, seg_len: torch.Tensor, slot: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = h[t] + (prev - h[t]) * mix: prev is the row before inside a request's segment and the request's
+    state at the segment's first token; the state then becomes the segment's last row of h."""
+    n, width = h.shape
+    n_rows = seg_start.shape[0]
+    _check(library().imparo_token_shift(
+        _dev(h, "normed rows", torch.float32), _dev(mix, "shift mix", torch.float32, (width,)),
+        _dev(state, "shift state", torch.float32, (state.shape[0], width)),
+        _dev(row_of_token, "row_of_token", torch.int32, (n,)), _dev(seg_start, "seg_start", torch.int32, (n_rows,)),
+        _dev(seg_len, "seg_len", torch.int32, (n_rows,)), _dev(slot, "slot", torch.int32, (n_rows,)),
+        _dev(out, "shifted rows", None, (n, width)), _code(out, "shifted rows"), n, n_rows, width, _stream()), "token_shift")
+    return out
+
+
+def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float, out: torch.Tensor, width: Optional[int] = None) -> torch.Tensor:
+    """out = a N(z) + b N(z^2) + c N(z^3) + e over the first `width` values of every row of z (default: all),
+    N(v) = v / sqrt(mean(v^2) + eps); coef = [a, b, c, e] on the device. Columns of out beyond `width` become zero."""
+    n, z_ld = z.shape
+    width = z_ld if width is None else int(width)
+    if out.shape[0] != n or out.dim() != 2 or out.shape[1] < width or width > z_ld:
+        raise KernelArgumentError("poly_norm: the output does not match the rows")
+    _check(library().imparo_poly_norm(
+        _dev(z, "poly_norm z", torch.float32), z_ld, _dev(coef, "poly_norm coefficients", torch.float32, (4,)),
+        _dev(out, "poly_norm out"), _code(out, "poly_norm out"), out.shape[1], n, width, float(eps), _stream()), "poly_norm")
+    return out
+
+
+# ------------------------------------------------------------------ selective state-space mixer
+def causal_conv(u: torch.Tensor, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                state: Optional[torch.Tensor], row_of_token: torch.Tensor, seg_start: torch.Tensor, seg_len: torch.Tensor,
+                slot: torch.Tensor, out: torch.Tensor, silu: bool = True, single_tokens: bool = False) -> torch.Tensor:
+    """Causal per-channel convolution of each request's segment over the first `channels` columns of u
+    (float32 rows), continued from the request's history, which is advanced: state [slots, taps - 1,
+    channels] (None with one tap). The last tap is the current token's."""
+    n, u_ld = u.shape
+    ch, taps = weight.shape
+    n_rows = seg_start.shape[0]
+    if ch != channels or u_ld < channels:
+        raise KernelArgumentError(f"causal_conv: a [{ch}, {taps}] filter does not fit {channels} channels of rows of {u_ld}")
+    if taps > 1:
+        if state is None:
+            raise KernelArgumentError("causal_conv: a filter of more than one tap needs a history")
+        _dev(state, "conv history", torch.float32, (state.shape[0], taps - 1, channels))
+    _check(library().imparo_causal_conv(
+        _dev(u, "conv input", torch.float32), u_ld, _dev(weight, "conv weight", torch.float32),
+        _dev(bias, "conv bias", torch.float32, (channels,)), _dev(state, "conv history", torch.float32) if taps > 1 else 0,
+        _dev(row_of_token, "row_of_token", torch.int32, (n,)), _dev(seg_start, "seg_start", torch.int32, (n_rows,)),
+        _dev(seg_len, "seg_len", torch.int32, (n_rows,)), _dev(slot, "slot", torch.int32, (n_rows,)),
+        _dev(out, "conv out", None, (n, channels)), _code(out, "conv out"), n, n_rows, channels, taps, int(silu),
+        int(single_tokens), _stream()), "causal_conv")
+    return out
+
+
+def selective_scan(dt_raw: torch.Tensor, x: torch.Tensor, bc: torch.Tensor, z: torch.Tensor, z_ld: int, A: torch.Tensor,
+                   D: torch.Tensor, state: torch.Tensor, seg_start: torch.Tensor, seg_len: torch.Tensor,
+                   slot: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """The selective scan of every request's segment, continued from its state [slots, channels, n_state]
+    (float32), which is advanced. dt_raw [tokens, channels] float32 before softplus; x and out [tokens,
+    channels] in one dtype; bc [tokens, 2 n_state] float32; z a float32 view whose rows lie z_ld apart."""
+    n, channels = x.shape
+    n_state = A.shape[1]
+    n_rows = seg_start.shape[0]
+    if z.dtype != torch.float32 or z.device != x.device or z_ld < channels:
+        raise KernelArgumentError("selective_scan: z is float32 on the GPU, its rows at least `channels` apart")
+    _check(library().imparo_selective_scan(
+        _dev(dt_raw, "dt", torch.float32, (n, channels)), _dev(x, "scan x"), _dev(bc, "B and C", torch.float32, (n, 2 * n_state)),
+        z.data_ptr(), int(z_ld), _dev(A, "A", torch.float32, (channels, n_state)), _dev(D, "D", torch.float32, (channels,)),
+        _dev(state, "scan state", torch.float32, (state.shape[0], channels, n_state)),
+        _dev(seg_start, "seg_start", torch.int32, (n_rows,)), _dev(seg_len, "seg_len", torch.int32, (n_rows,)),
+        _dev(slot, "slot", torch.int32, (n_rows,)), _dev(out, "scan out", x.dtype, (n, channels)), _code(x, "scan x"),
+        n_rows, channels, n_state, _stream()), "selective_scan")
+    return out
+
+
+# ------------------------------------------------------------------ differential attention
+def diff_attention_split() -> int:
+    """Keys per split of the differential attention kernel."""
+    return int(library().imparo_diff_attention_split())
+
+
+def diff_qkv_store(rows_in: torch.Tensor, positions: torch.Tensor, row_of_token: torch.Tensor,
+                   block_table: Optional[torch.Tensor], page_size: int, q_out: torch.Tensor,
+                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], heads: int, kv_heads: int, dim: int,
+                   vdim: int, temp_coef: float, temp_every: int) -> torch.Tensor:
+    """From the fused projection's float32 rows [q | k | v | ...]: the queries times their position's
+    temperature into q_out [tokens, heads, 2, dim]; keys and values into their pages (caches None: not written)."""
+    n, ld = rows_in.shape
+    write_kv = k_cache is not None
+    n_pages, stride = 0, 0
+    if write_kv:
+        n_pages = k_cache.shape[0]
+        _dev(k_cache, "k cache", q_out.dtype, (n_pages, 2 * kv_heads, page_size, dim))
+        _dev(v_cache, "v cache", q_out.dtype, (n_pages, kv_heads, page_size, vdim))
+        if block_table is None or block_table.dim() != 2:
+            raise KernelArgumentError("diff_qkv_store: a [rows, pages] block table is needed to write the cache")
+        stride = block_table.shape[1]
+    _check(library().imparo_diff_qkv_store(
+        _dev(rows_in, "projection rows", torch.float32), ld, _dev(positions, "positions", torch.int32, (n,)),
+        _dev(row_of_token, "row_of_token", torch.int32, (n,)), _dev(block_table, "block table", torch.int32) if write_kv else 0,
+        stride, page_size, _dev(q_out, "q out", None, (n, heads, 2, dim)), _dev(k_cache, "k cache"), _dev(v_cache, "v cache"),
+        _code(q_out, "q out"), int(write_kv), n, heads, kv_heads, dim, vdim, n_pages, float(temp_coef), int(temp_every),
+        _stream()), "diff_qkv_store")
+    return q_out
+
+
+def diff_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gate: Optional[torch.Tensor],
+                   gate_ld: int, out: torch.Tensor, positions: torch.Tensor, row_of_token: torch.Tensor,
+                   block_table: torch.Tensor, scale: float, window: Optional[int], lam: float, eps: float,
+                   out_scale: float, part: Optional[torch.Tensor] = None, n_splits: int = 1) -> torch.Tensor:
+    """Differential attention of every token over its request's cached keys (see imparo_diff_attention)."""
+    n, heads, two, dim = q.shape
+    n_pages, kv2, page_size, kdim = k_cache.shape
+    kv_heads, vdim = v_cache.shape[1], v_cache.shape[3]
+    if two != 2 or kdim != dim or kv2 != 2 * kv_heads or heads % kv_heads:
+        raise KernelArgumentError("diff_attention: queries [tokens, heads, 2, dim], keys [pages, 2 kv_heads, page, dim]")
+    _dev(v_cache, "v cache", q.dtype, (n_pages, kv_heads, page_size, vdim))
+    if n_splits > 1 and (part is None or part.numel() < n * heads * n_splits * (2 * vdim + 4)):
+        raise KernelArgumentError("diff_attention: the scratch for partial results is too small")
+    if gate is not None and (gate.dtype != torch.float32 or gate.device != q.device):
+        raise KernelArgumentError("diff_attention: the gate's logits are float32 on the GPU")
+    _check(library().imparo_diff_attention(
+        _dev(q, "q"), _dev(k_cache, "k cache", q.dtype), v_cache.data_ptr(), 0 if gate is None else gate.data_ptr(),
+        int(gate_ld), _dev(out, "attention out", q.dtype, (n, heads * vdim)), _dev(part, "partial results", torch.float32),
+        _code(q, "q"), _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
+        _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size, n, heads, kv_heads, dim, vdim,
+        n_pages, float(scale), int(window or 0), float(lam), float(eps), float(out_scale), int(n_splits), _stream()),
+        "diff_attention")
+    return out

@@ -3,37 +3,66 @@
 pre_norm: x += mixer(norm_a(x)); x += ffn(norm_b(x)) -- no post-norms
 (/root/reference/crates/imparo-model/src/lfm2/workflow_cpu.rs:8-15). Each
 delta is left pending on the residual stream so that the next norm, whichever
-block it belongs to, adds it while reading the row."""
+block it belongs to, adds it while reading the row.
+
+Two optional parts widen the arrangement: `shift` (role "shift") mixes what
+the mixer reads with the token before it and keeps the last token's input as
+state of the block's own, beside the mixer's; a layer without `ffn` and
+`ffn_norm` has no feed-forward."""
 from __future__ import annotations
 
 from typing import Dict
 
+import torch
+
+from ..cache.pages import with_fixed_arrays
 from .base import Residual, StepContext, emits
 from .registry import register_part
 
 
 class PreNormBlock:
-    """Reads four parts by name: mixer_norm, mixer, ffn_norm, ffn."""
+    """Reads its parts by name: mixer_norm, mixer, ffn_norm, ffn; optionally shift; ffn_norm and ffn may be absent."""
     role = "block"
     graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     def __init__(self, parts: Dict[str, object]):
         self.parts = parts
         self.mixer_norm, self.mixer = parts["mixer_norm"], parts["mixer"]
-        self.ffn_norm, self.ffn = parts["ffn_norm"], parts["ffn"]
+        self.ffn_norm, self.ffn = parts.get("ffn_norm"), parts.get("ffn")
+        self.shift = parts.get("shift")
+        if (self.ffn is None) != (self.ffn_norm is None):
+            raise ValueError("a block has a feed-forward and the norm before it, or neither")
 
     def cache_spec(self, page_size: int):
-        """What a call of this block keeps between steps: its mixer's state."""
-        return self.mixer.cache_spec(page_size)
+        """What a call of this block keeps between steps: its mixer's state and,
+        with a token shift, the input that the request's last token left."""
+        spec = self.mixer.cache_spec(page_size)
+        if self.shift is not None:
+            spec = with_fixed_arrays(spec, self.shift.state_arrays())
+        return spec
 
     def forward(self, ctx: StepContext, res: Residual, site: int, owns_cache: bool) -> None:
-        h = self.mixer_norm.forward(ctx, res, self.mixer.in_dtype)
+        if self.shift is None:
+            h = self.mixer_norm.forward(ctx, res, self.mixer.in_dtype)
+        elif not owns_cache:
+            raise ValueError("a token shift's state cannot be read from another layer")
+        elif ctx.max_seg_len == 1 and hasattr(self.mixer_norm, "forward_shifted"):
+            # every row brings one token: the shift rides in the norm's launch
+            h = self.mixer_norm.forward_shifted(ctx, res, self.mixer.in_dtype, self.shift.mix,
+                                                self.shift.state(ctx, site))
+        else:
+            h = self.shift.forward(ctx, site, self.mixer_norm.forward(ctx, res, torch.float32, name="normed_f32"),
+                                   self.mixer.in_dtype)
         res.pending = self._delta(ctx, res, lambda: self.mixer.forward(ctx, site, owns_cache, h))
-        n = self.ffn_norm.forward(ctx, res, self.ffn.in_dtype)
-        res.pending = self._delta(ctx, res, lambda: self.ffn.forward(ctx, n))
+        if self.ffn is not None:
+            n = self.ffn_norm.forward(ctx, res, self.ffn.in_dtype)
+            res.pending = self._delta(ctx, res, lambda: self.ffn.forward(ctx, n))
 
     def can_emit(self) -> bool:
-        return all(emits(p) for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
+        if self.shift is not None or self.ffn is None:
+            return False          # the step program knows the four-part block only
+        parts = (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+        return all(emits(p) and getattr(p, "can_emit", lambda: True)() for p in parts)
 
     def emit(self, program, site: int, owns_cache: bool) -> None:
         """Appends `forward` to a native step program: the four parts in the order they run."""

@@ -1,11 +1,17 @@
 """Token embedding (a row gather, no scale:
 /root/reference/crates/imparo-model/src/cpu_support.rs:327-342) and the output
 head (logits = W h for the rows that want logits, no bias, no softcap:
-/root/reference/crates/imparo-model/src/cpu_support.rs:451-466)."""
+/root/reference/crates/imparo-model/src/cpu_support.rs:451-466).
+
+`tensor` names the table outright where a checkpoint does not call it
+`<prefix>.weight`. The sinusoidal embedding adds a position vector to the
+gathered row: entry 2i is sin(p * base^(-2i/width)), entry 2i+1 the cosine of
+the same angle, angles in float32."""
 from __future__ import annotations
 
 from typing import Dict
 
+import numpy as np
 import torch
 
 from ..config.plan import PartSpec
@@ -16,17 +22,21 @@ from .linear import Linear, place_matrix
 from .registry import register_part
 
 
+def _table_name(spec: PartSpec) -> str:
+    return spec.get("tensor") or f"{spec.prefix}.weight"
+
+
 class Embedding:
     role = "embedding"
     graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     @staticmethod
     def declare(spec: PartSpec) -> Declared:
-        return {f"{spec.prefix}.weight": (TensorDecl((spec["vocab"], spec["width"])), "matrix")}
+        return {_table_name(spec): (TensorDecl((spec["vocab"], spec["width"])), "matrix")}
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
                  engine_dtype: torch.dtype, placed: Dict[str, torch.Tensor]):
-        name = f"{spec.prefix}.weight"
+        name = _table_name(spec)
         if name not in placed:     # a tied head shares this very tensor
             placed[name] = place_matrix(tensors[name], engine_dtype, device)
         self.table = placed[name]
@@ -41,17 +51,33 @@ class Embedding:
         program.embedding(self.table, self.vocab, self.width)
 
 
+class SinusoidEmbedding(Embedding):
+    """The table's row plus the sinusoidal vector of the token's position."""
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
+                 engine_dtype: torch.dtype, placed: Dict[str, torch.Tensor]):
+        super().__init__(spec, tensors, device, engine_dtype, placed)
+        base = float(spec.get("base") or 10000.0)
+        i = np.arange((self.width + 1) // 2, dtype=np.float32)
+        expo = (np.float32(-2.0) * i / np.float32(self.width)).astype(np.float32)
+        self.inv_freq = torch.from_numpy(np.power(np.float32(base), expo).astype(np.float32)).to(device)
+
+    def forward(self, ctx: StepContext, token_ids: torch.Tensor) -> torch.Tensor:
+        x = ctx.workspace.get("residual", (token_ids.shape[0], self.width), torch.float32)
+        return ops.embed_sinusoid(self.table, token_ids, ctx.positions, self.inv_freq, x)
+
+
 class LinearHead:
     role = "head"
     graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     @staticmethod
     def declare(spec: PartSpec) -> Declared:
-        return {f"{spec.prefix}.weight": (TensorDecl((spec["vocab"], spec["width"])), "matrix")}
+        return {_table_name(spec): (TensorDecl((spec["vocab"], spec["width"])), "matrix")}
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
                  engine_dtype: torch.dtype, placed: Dict[str, torch.Tensor]):
-        name = f"{spec.prefix}.weight"
+        name = _table_name(spec)
         if name not in placed:
             placed[name] = place_matrix(tensors[name], engine_dtype, device)
         self.proj = Linear(placed[name])
@@ -70,4 +96,5 @@ class LinearHead:
 
 
 register_part("embedding", "embedding", Embedding)
+register_part("embedding", "sinusoid_embedding", SinusoidEmbedding)
 register_part("head", "linear_head", LinearHead)

@@ -1,5 +1,10 @@
 """Dense SwiGLU feed-forward: f = W2 ( silu(W1 n) * (W3 n) ), SiLU on the gate
-(/root/reference/crates/imparo-model/src/lfm2/workflow_cpu.rs:298-316)."""
+(/root/reference/crates/imparo-model/src/lfm2/workflow_cpu.rs:298-316).
+
+PolyNorm feed-forward: f = Wdown act(Wup n) with act(z) = a N(z) + b N(z^2) +
+c N(z^3) + e, powers taken element by element and N dividing a token's vector
+of hidden values by its root mean square (in float32); a, b, c, e are four
+numbers of the layer."""
 from __future__ import annotations
 
 from typing import Dict
@@ -7,9 +12,10 @@ from typing import Dict
 import torch
 
 from ..config.plan import PartSpec
+from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .base import Declared, StepContext
-from .linear import Linear, place_matrix
+from .linear import Linear, place_matrix, place_vector
 from .registry import register_part
 
 _DEFAULT_NAMES = dict(gate="gate_proj", up="up_proj", down="down_proj")
@@ -74,4 +80,52 @@ class SwiGlu:
         program.swiglu(SwigluDesc(program.linear(self.gate_up), program.linear(self.down)))
 
 
+class PolyNormFfn:
+    role = "feed_forward"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
+
+    @staticmethod
+    def _names(spec: PartSpec) -> Dict[str, str]:
+        names = dict(up="up", down="down", act="act")
+        names.update(spec.get("names") or {})
+        return {k: f"{spec.prefix}.{v}" for k, v in names.items()}
+
+    @classmethod
+    def declare(cls, spec: PartSpec) -> Declared:
+        n = cls._names(spec)
+        E, F = spec["width"], spec["hidden"]
+        return {
+            n["up"]: (TensorDecl((F, E)), "matrix"),
+            n["down"]: (TensorDecl((E, F)), "matrix"),
+            n["act"]: (TensorDecl((4,), "vector"), "wide"),
+        }
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
+                 engine_dtype: torch.dtype):
+        n = self._names(spec)
+        self.width, self.hidden = spec["width"], spec["hidden"]
+        self.eps = float(spec["eps"])
+        up, down = tensors[n["up"]], tensors[n["down"]]
+        # a hidden width that is no multiple of 8 is filled up with units of zero weight on the way back
+        # (the bfloat16 kernels walk K in steps of 8); the norms divide by the true width
+        fill = (-self.hidden) % 8
+        if fill and engine_dtype != torch.float32 and down.dtype != torch.float32:
+            up = torch.cat([up, up.new_zeros(fill, self.width)])
+            down = torch.cat([down, down.new_zeros(self.width, fill)], dim=1)
+        self.up = Linear(place_matrix(up, engine_dtype, device))
+        self.down = Linear(place_matrix(down, engine_dtype, device))
+        self.coef = place_vector(tensors[n["act"]], device)
+
+    @property
+    def in_dtype(self) -> torch.dtype:
+        return self.up.in_dtype
+
+    def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
+        z = self.up(ctx, n, torch.float32, "ffn_hidden", alias="mixer_in")
+        g = ctx.workspace.get("ffn_act", tuple(z.shape), self.down.in_dtype, alias="mixer_mid")
+        ops.poly_norm(z, self.coef, self.eps, g, width=self.hidden)
+        return self.down(ctx, g, torch.float32, "ffn_out", sliced_ok=True, into=ctx.stream)
+
+
 register_part("feed_forward", "swiglu", SwiGlu)
+register_part("feed_forward", "poly_norm", PolyNormFfn)

@@ -1,7 +1,12 @@
 """RMS norm: y = x * rsqrt(mean(x^2) + eps) * w, no offset, no bias
 (/root/reference/crates/imparo-cpu/src/ops.rs:6-22). The residual add that
 precedes a norm is fused into it (the reference's add_rms_norm,
-/root/reference/crates/imparo-backend/src/lib.rs:2603-2609)."""
+/root/reference/crates/imparo-backend/src/lib.rs:2603-2609).
+
+With `groups` > 1 the row is cut into that many equal consecutive parts and
+each is divided by its own root mean square; the weight spans the whole row.
+`tensor` names the weight outright where a checkpoint does not call it
+`<prefix>.weight`."""
 from __future__ import annotations
 
 from typing import Dict
@@ -21,28 +26,53 @@ class RmsNorm:
     graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     @staticmethod
-    def declare(spec: PartSpec) -> Declared:
-        return {f"{spec.prefix}.weight": (TensorDecl((spec["width"],), "vector"), "norm")}
+    def _tensor(spec: PartSpec) -> str:
+        return spec.get("tensor") or f"{spec.prefix}.weight"
+
+    @classmethod
+    def declare(cls, spec: PartSpec) -> Declared:
+        return {cls._tensor(spec): (TensorDecl((spec["width"],), "vector"), "norm")}
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
                  engine_dtype: torch.dtype):
         self.width = spec["width"]
         self.eps = float(spec["eps"])
-        self.weight = place_vector(tensors[f"{spec.prefix}.weight"], device)
+        self.groups = int(spec.get("groups") or 1)
+        if self.groups < 1 or self.width % self.groups:
+            raise ValueError(f"a norm over {self.width} values cannot be cut into {self.groups} equal parts")
+        self.weight = place_vector(tensors[self._tensor(spec)], device)
 
     def forward(self, ctx: StepContext, res: Residual, out_dtype: torch.dtype, name: str = "normed") -> torch.Tensor:
         """Adds the pending delta into the stream (if any) and returns the
         normed rows in `out_dtype`."""
         out = ctx.workspace.get(name, tuple(res.x.shape), out_dtype)
-        if res.pending is not None:
-            ops.rms_norm(res.x, self.weight, self.eps, out, delta=res.pending, write_back=True)
-            res.pending = None
+        pending, res.pending = res.pending, None
+        if self.groups > 1:
+            ops.group_rms_norm(res.x, self.weight, self.groups, self.eps, out, delta=pending,
+                               write_back=pending is not None)
+        elif pending is not None:
+            ops.rms_norm(res.x, self.weight, self.eps, out, delta=pending, write_back=True)
         else:
             ops.rms_norm(res.x, self.weight, self.eps, out)
         return out
 
+    def forward_shifted(self, ctx: StepContext, res: Residual, out_dtype: torch.dtype, mix: torch.Tensor,
+                        state: torch.Tensor, name: str = "normed") -> torch.Tensor:
+        """`forward` for a step whose rows all bring one token, with the token shift behind the norm in
+        the same launch: out = h + (prev - h) * mix, where the request's prev (state[slot]) becomes h."""
+        out = ctx.workspace.get(name, tuple(res.x.shape), out_dtype)
+        pending, res.pending = res.pending, None
+        ops.group_rms_norm(res.x, self.weight, self.groups, self.eps, out, delta=pending,
+                           write_back=pending is not None, shift_mix=mix, shift_state=state, slot=ctx.slot)
+        return out
+
+    def can_emit(self) -> bool:
+        return self.groups == 1
+
     def emit(self, program, out_dtype: torch.dtype) -> None:
         """Appends `forward` to a native step program."""
+        if self.groups != 1:
+            raise ValueError("the step program's norm does not cut rows into groups")
         program.norm(self.weight, self.eps, self.width, out_dtype)
 
     def emit_head(self, program, head_linear) -> None:
@@ -54,7 +84,10 @@ class RmsNorm:
         """Norm of selected rows only (the rows whose logits are wanted); the
         stream itself is left as it is."""
         out = ctx.workspace.get(name, (rows.shape[0], self.width), out_dtype)
-        ops.rms_norm(res.x, self.weight, self.eps, out, delta=res.pending, rows=rows)
+        if self.groups > 1:
+            ops.group_rms_norm(res.x, self.weight, self.groups, self.eps, out, delta=res.pending, rows=rows)
+        else:
+            ops.rms_norm(res.x, self.weight, self.eps, out, delta=res.pending, rows=rows)
         return out
 
 

@@ -3,7 +3,9 @@
 Every tensor is drawn from its own generator, seeded by (seed, tensor name),
 so the folder does not depend on the order tensors are declared in. The
 distributions: matrices and embeddings N(0, 0.02); depthwise conv taps
-N(0, 0.1); norm weights 1 + U(-0.1, 0.1); biases N(0, 0.02).
+N(0, 0.1); norm weights 1 + U(-0.1, 0.1); biases N(0, 0.02); a few numbers
+of a layer that act as they are (an activation's coefficients, the logarithms
+of decays: "wide") N(0, 0.5).
 """
 from __future__ import annotations
 
@@ -30,7 +32,7 @@ def random_tensor(seed: int, name: str, decl: TensorDecl, init: str) -> torch.Te
     g = _generator(seed, name)
     if init == "norm":
         return 1.0 + (torch.rand(decl.shape, generator=g) * 0.2 - 0.1)
-    std = 0.1 if init == "conv" else 0.02
+    std = {"conv": 0.1, "wide": 0.5}.get(init, 0.02)
     return torch.randn(decl.shape, generator=g) * std
 
 
