@@ -15,6 +15,7 @@ measurements taken in turn.
 """
 import argparse
 import json
+import math
 import os
 import sys
 import tempfile
@@ -387,6 +388,59 @@ def long_workload(dtype, requests, prompt_len, portion=2048, quiet=False, engine
                    "cache_pages_used": pages_used}}
 
 
+def tumadra_shape(width, heads, kv_heads, ff, inner, layers=16, attention_at=(2, 5, 8, 10, 12, 14)):
+    """A Tumadra model laid out like the LFM2 shapes above and of their size: differential attention where
+    they have attention (two maps of 64 a head, values of 128: the same q, k, v and output widths as their
+    heads of 64), a selective scan where they have a short conv (inner chosen so that the mixer's matrices
+    weigh what the conv block's do), a dense PolyNorm feed-forward with the parameters of their SwiGLU."""
+    attention = dict(heads=heads, kv_heads=kv_heads, dim=64, vdim=128, scale=0.125, diff=0.6,
+                     q_temp=dict(coef=0.3, every=256))
+    scan = dict(inner=inner, state=16, dt_rank=width // 16, conv=4)
+    mlp = dict(kind="dense", ff=ff)
+    return dict(architecture="Tumadra", vocab=65536, width=width, norm=dict(eps=1e-5, groups=4),
+                layers=[dict(type="attention" if i in attention_at else "mamba1",
+                             mixer=attention if i in attention_at else scan, mlp=mlp) for i in range(layers)])
+
+
+def tumadra_workload(dtype, steps, warmup):
+    """Prefill and decode throughput of the Tumadra design at two sizes, beside LFM2 (the closest model
+    the engine has: a hybrid of attention and a fixed-state mixer) at equal size, through the same loops."""
+    import torch
+    from imparo_amd.engine.model import declared_tensors
+    from imparo_amd.sampling import Sampler
+    sizes = [
+        ("1.2B", LFM2_1_2B, tumadra_shape(2048, 16, 4, 12288, 2816)),
+        ("350M", LFM2_350M, tumadra_shape(1024, 8, 4, 6912, 1408)),
+    ]
+    out = {"workload": "tumadra", "dtype": dtype, "data": "synthetic token ids, random weights", "sizes": []}
+    for name, lfm2, tumadra in sizes:
+        row = {"size": name}
+        for label, cfg in (("lfm2", lfm2), ("tumadra", tumadra)):
+            print(f"[bench] {name} {label}: writing random weights ...", file=sys.stderr, flush=True)
+            engine = build_engine(cfg, 2, dtype, max_tokens=8 * (4096 + 64) + 8192 + 64, max_requests=8,
+                                  max_step_tokens=8192)
+            sampler = Sampler(engine.device)
+            vocab = engine.vocab_size
+            params = sum(math.prod(d.shape) for d, _ in declared_tensors(engine.plan).values())
+            r = {"parameters_B": round(params / 1e9, 3), "native_step_program": engine.program is not None}
+            for tokens in (512, 2048, 8192):
+                t = median(prefill_run(engine, tokens, vocab, 3, 3))
+                r[f"prefill_{tokens}_tok_s"] = round(tokens / t, 1)
+                r[f"prefill_{tokens}_ms"] = round(t * 1e3, 3)
+            for batch, context in ((1, 4096), (8, 4096)):
+                dt = median([decode_run(engine, sampler, batch, context, steps, warmup, vocab, 5 + i) for i in range(3)])
+                r[f"decode_b{batch}_ctx{context}_tok_s"] = round(batch * steps / dt, 1)
+                r[f"decode_b{batch}_ctx{context}_ms_per_step"] = round(dt / steps * 1e3, 4)
+            row[label] = r
+            del engine, sampler
+            torch.cuda.empty_cache()
+        for key in list(row["tumadra"]):
+            if key.endswith("tok_s"):
+                row.setdefault("tumadra_over_lfm2", {})[key] = round(row["tumadra"][key] / row["lfm2"][key], 3)
+        out["sizes"].append(row)
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -398,10 +452,11 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="run only the 2,048-token prefill (for profiling)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "long"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "long", "tumadra"],
                     help="decode: the headline line (default). serving: continuous batching of 32 requests in 4 "
                          "waves (LFM2-700M shape). long: 64 requests of 32,768-token prompts, then 128 tokens "
-                         "each (LFM2-350M shape). The last two print a line of their own")
+                         "each (LFM2-350M shape). tumadra: prefill and decode of the Tumadra design at two sizes "
+                         "beside LFM2 at equal size. The last three print a line of their own")
     ap.add_argument("--requests", type=int, default=64, help="--workload long: concurrent requests")
     ap.add_argument("--prompt-len", type=int, default=32768, help="--workload long: tokens per prompt")
     ap.add_argument("--portion", type=int, default=2048, help="--workload long: tokens of a prompt per step")
@@ -414,6 +469,9 @@ def main() -> int:
         return 0
     if args.workload == "long":
         print(json.dumps(long_workload(args.dtype, args.requests, args.prompt_len, args.portion)), flush=True)
+        return 0
+    if args.workload == "tumadra":
+        print(json.dumps(tumadra_workload(args.dtype, args.steps, args.warmup)), flush=True)
         return 0
 
     import torch

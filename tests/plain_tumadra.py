@@ -64,6 +64,35 @@ def token_shift(h: torch.Tensor, mix: torch.Tensor) -> torch.Tensor:
     return h + (before - h) * mix
 
 
+def query_temperature(positions: torch.Tensor, coef: float, every: int, dtype=torch.float32) -> torch.Tensor:
+    """1 + coef * ln(floor((p + 1) / every) + 1)."""
+    return 1.0 + coef * torch.log(torch.floor((positions + 1) / every).to(dtype) + 1.0)
+
+
+def differential_core(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_pos: torch.Tensor, scale: float,
+                      lam: float, diff: float, eps: float) -> torch.Tensor:
+    """q [Tq, H, 2, D] at positions q_pos, k [Tk, G, 2, D] and v [Tk, G, V] at positions 0..Tk-1:
+    per head a1 - lam a2 over the keys j <= q_pos, divided by its root mean square, times 1 - diff.
+    Returns [Tq, H * V]."""
+    Tq, H = q.shape[0], q.shape[1]
+    Tk, G = k.shape[0], k.shape[1]
+    seen = torch.arange(Tk)[None, :] <= q_pos[:, None]
+    heads = []
+    for head in range(H):
+        g = head // (H // G)
+        maps = []
+        for m in range(2):
+            s = (q[:, head, m] @ k[:, g, m].T) * scale
+            s = s.masked_fill(~seen, float("-inf"))
+            maps.append(torch.softmax(s, dim=-1) @ v[:, g])
+        heads.append(rms(maps[0] - lam * maps[1], eps) * (1.0 - diff))
+    return torch.cat(heads, dim=-1)
+
+
+def differential_lambda(p: Dict[str, torch.Tensor], diff: float) -> float:
+    return float(torch.exp((p["lq1"] * p["lk1"]).sum()) - torch.exp((p["lq2"] * p["lk2"]).sum()) + diff)
+
+
 def differential_attention(h: torch.Tensor, p: Dict[str, torch.Tensor], c: dict, eps: float) -> torch.Tensor:
     """Two softmax maps per head over shared values, a1 - lambda a2, unit-RMS
     per head times (1 - diff), a sigmoid gate, the output projection."""
@@ -73,47 +102,47 @@ def differential_attention(h: torch.Tensor, p: Dict[str, torch.Tensor], c: dict,
     k = (h @ p["k"].T + p["k.b"]).reshape(T, G, 2, D)
     v = (h @ p["v"].T + p["v.b"]).reshape(T, G, V)
     pos = torch.arange(T)
-    temp = 1.0 + c["q_temp"]["coef"] * torch.log(torch.floor((pos + 1) / c["q_temp"]["every"]).to(h.dtype) + 1.0)
-    q = q * temp.to(h.dtype)[:, None, None, None]
-    lam = torch.exp((p["lq1"] * p["lk1"]).sum()) - torch.exp((p["lq2"] * p["lk2"]).sum()) + c["diff"]
-    causal = pos[None, :] <= pos[:, None]
-    heads = []
-    for head in range(H):
-        g = head // (H // G)
-        maps = []
-        for m in range(2):
-            s = (q[:, head, m] @ k[:, g, m].T) * c["scale"]
-            s = s.masked_fill(~causal, float("-inf"))
-            maps.append(torch.softmax(s, dim=-1) @ v[:, g])
-        o = maps[0] - lam * maps[1]
-        heads.append(rms(o, eps) * (1.0 - c["diff"]))
-    o = torch.cat(heads, dim=-1) * torch.sigmoid(h @ p["g"].T)
-    return o @ p["o"].T
+    if c.get("q_temp"):
+        q = q * query_temperature(pos, c["q_temp"]["coef"], c["q_temp"]["every"], h.dtype)[:, None, None, None]
+    o = differential_core(q, k, v, pos, c["scale"], differential_lambda(p, c["diff"]), c["diff"], eps)
+    return (o * torch.sigmoid(h @ p["g"].T)) @ p["o"].T
+
+
+def causal_conv(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """out[t, c] = b[c] + sum_j w[c, j] x[t - (taps - 1) + j, c], zeros before the start."""
+    T, C = x.shape
+    taps = w.shape[1]
+    padded = torch.cat([torch.zeros(taps - 1, C, dtype=x.dtype), x], dim=0)
+    out = b.expand(T, C).clone()
+    for j in range(taps):
+        out = out + padded[j:j + T] * w[:, j]
+    return out
+
+
+def scan(dt: torch.Tensor, x: torch.Tensor, B: torch.Tensor, C: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
+         S: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """S <- exp(dt A) S + dt x B; y = S C + D x, token by token from S = 0 (or the given S, updated in place)."""
+    T, inner = x.shape
+    if S is None:
+        S = torch.zeros(inner, A.shape[1], dtype=x.dtype)
+    ys = []
+    for t in range(T):
+        S.copy_(torch.exp(dt[t][:, None] * A) * S + (dt[t] * x[t])[:, None] * B[t][None, :])
+        ys.append(S @ C[t] + D * x[t])
+    return torch.stack(ys)
 
 
 def mamba1(h: torch.Tensor, p: Dict[str, torch.Tensor], c: dict) -> torch.Tensor:
     """Selective scan: in -> (x, z); x through a causal per-channel conv and
     silu; (dt, B, C) from x; S <- exp(dt A) S + dt x B; y = S C + D x; y silu(z); out."""
-    T = h.shape[0]
-    inner, N, R, taps = c["inner"], c["state"], c["dt_rank"], c["conv"]
+    inner, N, R = c["inner"], c["state"], c["dt_rank"]
     xz = h @ p["in"].T
     x, z = xz[:, :inner], xz[:, inner:]
-    padded = torch.cat([torch.zeros(taps - 1, inner, dtype=h.dtype), x], dim=0)
-    conv = p["conv.b"].expand(T, inner).clone()
-    for j in range(taps):
-        conv = conv + padded[j:j + T] * p["conv"][:, j]
-    x = torch.nn.functional.silu(conv)
+    x = torch.nn.functional.silu(causal_conv(x, p["conv"], p["conv.b"]))
     low = x @ p["x"].T
     dt = torch.nn.functional.softplus(low[:, :R] @ p["dt"].T + p["dt.b"])
-    B, C = low[:, R:R + N], low[:, R + N:R + 2 * N]
-    A = -torch.exp(p["A_log"])
-    S = torch.zeros(inner, N, dtype=h.dtype)
-    ys = []
-    for t in range(T):
-        S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * x[t])[:, None] * B[t][None, :]
-        ys.append(S @ C[t] + p["D"] * x[t])
-    y = torch.stack(ys) * torch.nn.functional.silu(z)
-    return y @ p["o"].T
+    y = scan(dt, x, low[:, R:R + N], low[:, R + N:R + 2 * N], -torch.exp(p["A_log"]), p["D"])
+    return (y * torch.nn.functional.silu(z)) @ p["o"].T
 
 
 def poly_norm_ffn(n: torch.Tensor, p: Dict[str, torch.Tensor], eps: float) -> torch.Tensor:
@@ -142,7 +171,7 @@ class PlainTumadra:
         self.t = {k: v.to(dtype) for k, v in raw.items()}
         self.dtype = dtype
         self.eps = float(self.config["norm"]["eps"])
-        self.groups = int(self.config["norm"]["groups"])
+        self.groups = int(self.config["norm"].get("groups", 1))
 
     def _sub(self, prefix: str) -> Dict[str, torch.Tensor]:
         return {k[len(prefix):]: v for k, v in self.t.items() if k.startswith(prefix)}
