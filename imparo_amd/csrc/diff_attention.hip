@@ -18,7 +18,6 @@
 #define DA_WAVES 4
 #define DA_MAX_DIM 256
 #define DA_MAX_VDIM 512
-#define DA_DPL (DA_MAX_VDIM / WAVE)
 #define DA_SPLIT 256
 
 extern "C" int imparo_diff_attention_split(void) { return DA_SPLIT; }
@@ -92,14 +91,14 @@ __device__ __forceinline__ float da_dot<bf16_t>(const float* __restrict__ q, con
 
 // What finishes a head: o = a1 - lambda a2 over the head's vdim values (lane d holds d, d + 64, ...), divided
 // by its root mean square, times out_scale, times sigmoid(gate).
-template <typename T>
-__device__ __forceinline__ void da_finish(const float (&a1)[DA_DPL], const float (&a2)[DA_DPL], float lambda, float eps,
+template <typename T, int VPL>
+__device__ __forceinline__ void da_finish(const float (&a1)[VPL], const float (&a2)[VPL], float lambda, float eps,
                                           float out_scale, const float* __restrict__ gate, T* __restrict__ dst, int vdim,
                                           int lane) {
-    float o[DA_DPL];
+    float o[VPL];
     float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < DA_DPL; ++j) {
+    for (int j = 0; j < VPL; ++j) {
         const int d = lane + j * WAVE;
         o[j] = d < vdim ? a1[j] - lambda * a2[j] : 0.f;
         ss += o[j] * o[j];
@@ -107,7 +106,7 @@ __device__ __forceinline__ void da_finish(const float (&a1)[DA_DPL], const float
     ss = wave_sum(ss);
     const float r = out_scale / sqrtf(ss / (float)vdim + eps);
 #pragma unroll
-    for (int j = 0; j < DA_DPL; ++j) {
+    for (int j = 0; j < VPL; ++j) {
         const int d = lane + j * WAVE;
         if (d < vdim) {
             float y = o[j] * r;
@@ -117,7 +116,8 @@ __device__ __forceinline__ void da_finish(const float (&a1)[DA_DPL], const float
     }
 }
 
-template <typename T>
+// VPL: value dimensions a lane holds (d = lane, lane + 64, ...): vdim <= 64 VPL.
+template <typename T, int VPL>
 __global__ void k_diff_attention(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                  const float* __restrict__ gate, int gate_ld, T* __restrict__ out,
                                  float* __restrict__ part, const int32_t* __restrict__ positions,
@@ -152,9 +152,9 @@ __global__ void k_diff_attention(const T* __restrict__ q, const T* __restrict__ 
     for (int i = lane; i < 2 * dim; i += WAVE) qr[i] = load_f32<T>(qsrc, i);
     wave_lds_sync();
 
-    float a1[DA_DPL], a2[DA_DPL];
+    float a1[VPL], a2[VPL];
 #pragma unroll
-    for (int j = 0; j < DA_DPL; ++j) a1[j] = a2[j] = 0.f;
+    for (int j = 0; j < VPL; ++j) a1[j] = a2[j] = 0.f;
     float m1 = -INFINITY, l1 = 0.f, m2 = -INFINITY, l2 = 0.f;
 
     for (int c = first; c <= last; c += WAVE) {
@@ -187,22 +187,35 @@ __global__ void k_diff_attention(const T* __restrict__ q, const T* __restrict__ 
         wave_lds_sync();
         const int n_keys = min(WAVE, last - c + 1);
 #pragma unroll
-        for (int j = 0; j < DA_DPL; ++j) {
+        for (int j = 0; j < VPL; ++j) {
             a1[j] *= c1;
             a2[j] *= c2;
         }
-        for (int kk = 0; kk < n_keys; ++kk) {
-            const long long vo = v_off[wave][kk];
-            if (vo < 0) continue;                 // uniform over the wave
-            const float w1 = probs[wave][0][kk], w2 = probs[wave][1][kk];
-            const T* vrow = v_cache + vo;
+        // eight keys' values are asked for before any is used, from addresses that always lie in the cache
+        // (a key that is not there reads row 0 and weighs nothing); the sums run in the order of the keys
+        for (int kk0 = 0; kk0 < n_keys; kk0 += 8) {
+            float vals[8][VPL], w1[8], w2[8];
 #pragma unroll
-            for (int j = 0; j < DA_DPL; ++j) {
-                const int d = lane + j * WAVE;
-                if (d < vdim) {
-                    const float v = load_f32<T>(vrow, d);
-                    a1[j] += w1 * v;
-                    a2[j] += w2 * v;
+            for (int u = 0; u < 8; ++u) {
+                const int kk = min(kk0 + u, WAVE - 1);
+                const long long vo = v_off[wave][kk];
+                const bool on = kk0 + u < n_keys && vo >= 0;
+                const T* vrow = v_cache + (on ? vo : 0);
+                w1[u] = on ? probs[wave][0][kk] : 0.f;
+                w2[u] = on ? probs[wave][1][kk] : 0.f;
+#pragma unroll
+                for (int j = 0; j < VPL; ++j) {
+                    const int d = lane + j * WAVE;
+                    const float v = load_f32<T>(vrow, min(d, vdim - 1));
+                    vals[u][j] = on && d < vdim ? v : 0.f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+#pragma unroll
+                for (int j = 0; j < VPL; ++j) {
+                    a1[j] += w1[u] * vals[u][j];
+                    a2[j] += w2[u] * vals[u][j];
                 }
             }
         }
@@ -217,7 +230,7 @@ __global__ void k_diff_attention(const T* __restrict__ q, const T* __restrict__ 
             dst[3] = l2;
         }
 #pragma unroll
-        for (int j = 0; j < DA_DPL; ++j) {
+        for (int j = 0; j < VPL; ++j) {
             const int d = lane + j * WAVE;
             if (d < vdim) {
                 dst[4 + d] = a1[j];
@@ -228,16 +241,16 @@ __global__ void k_diff_attention(const T* __restrict__ q, const T* __restrict__ 
     }
     const float i1 = l1 > 0.f ? 1.0f / l1 : 0.f, i2 = l2 > 0.f ? 1.0f / l2 : 0.f;
 #pragma unroll
-    for (int j = 0; j < DA_DPL; ++j) {
+    for (int j = 0; j < VPL; ++j) {
         a1[j] *= i1;
         a2[j] *= i2;
     }
-    da_finish<T>(a1, a2, lambda, eps, out_scale, gate ? gate + (size_t)t * gate_ld + (size_t)h * vdim : nullptr,
+    da_finish<T, VPL>(a1, a2, lambda, eps, out_scale, gate ? gate + (size_t)t * gate_ld + (size_t)h * vdim : nullptr,
                  out + ((size_t)t * heads + h) * vdim, vdim, lane);
 }
 
 // One wave per (token, head): the splits that hold keys of the query, in order.
-template <typename T>
+template <typename T, int VPL>
 __global__ void k_diff_merge(const float* __restrict__ part, const float* __restrict__ gate, int gate_ld,
                              T* __restrict__ out, const int32_t* __restrict__ positions, int n_tokens, int heads,
                              int vdim, int window, float lambda, float eps, float out_scale, int n_splits) {
@@ -256,9 +269,9 @@ __global__ void k_diff_merge(const float* __restrict__ part, const float* __rest
         m1 = fmaxf(m1, p[0]);
         m2 = fmaxf(m2, p[2]);
     }
-    float a1[DA_DPL], a2[DA_DPL];
+    float a1[VPL], a2[VPL];
 #pragma unroll
-    for (int j = 0; j < DA_DPL; ++j) a1[j] = a2[j] = 0.f;
+    for (int j = 0; j < VPL; ++j) a1[j] = a2[j] = 0.f;
     float l1 = 0.f, l2 = 0.f;
     for (int s = s_first; s <= s_last; ++s) {
         const float* p = base + (size_t)s * (2 * vdim + 4);
@@ -267,7 +280,7 @@ __global__ void k_diff_merge(const float* __restrict__ part, const float* __rest
         l1 += w1 * p[1];
         l2 += w2 * p[3];
 #pragma unroll
-        for (int j = 0; j < DA_DPL; ++j) {
+        for (int j = 0; j < VPL; ++j) {
             const int d = lane + j * WAVE;
             if (d < vdim) {
                 a1[j] += w1 * p[4 + d];
@@ -277,11 +290,11 @@ __global__ void k_diff_merge(const float* __restrict__ part, const float* __rest
     }
     const float i1 = l1 > 0.f ? 1.0f / l1 : 0.f, i2 = l2 > 0.f ? 1.0f / l2 : 0.f;
 #pragma unroll
-    for (int j = 0; j < DA_DPL; ++j) {
+    for (int j = 0; j < VPL; ++j) {
         a1[j] *= i1;
         a2[j] *= i2;
     }
-    da_finish<T>(a1, a2, lambda, eps, out_scale, gate ? gate + (size_t)t * gate_ld + (size_t)h * vdim : nullptr,
+    da_finish<T, VPL>(a1, a2, lambda, eps, out_scale, gate ? gate + (size_t)t * gate_ld + (size_t)h * vdim : nullptr,
                  out + ((size_t)t * heads + h) * vdim, vdim, lane);
 }
 
@@ -331,37 +344,37 @@ extern "C" int imparo_diff_attention(const void* q, const void* k_cache, const v
     if (blocks > 0x7fffffffLL) return IMPARO_BAD_ARGUMENT;
     hipStream_t s = (hipStream_t)stream;
     const unsigned merge_blocks = (unsigned)(((long long)n_tokens * heads + DA_WAVES - 1) / DA_WAVES);
-    if (dtype == IMPARO_F32) {
-        k_diff_attention<float><<<(unsigned)blocks, DA_WAVES * WAVE, 0, s>>>(
-            (const float*)q, (const float*)k_cache, (const float*)v_cache, gate, gate_ld, (float*)out, part, positions,
-            row_of_token, block_table, table_stride, page_size, n_tokens, heads, kv_heads, dim, vdim, n_pages, scale,
-            window, lambda, eps, out_scale, n_splits);
-        if (n_splits > 1) {
-            if (launch_status()) return IMPARO_LAUNCH_FAILED;
-            k_diff_merge<float><<<merge_blocks, DA_WAVES * WAVE, 0, s>>>(part, gate, gate_ld, (float*)out, positions,
-                                                                         n_tokens, heads, vdim, window, lambda, eps,
-                                                                         out_scale, n_splits);
-        }
-    } else if (dtype == IMPARO_BF16) {
-        k_diff_attention<bf16_t><<<(unsigned)blocks, DA_WAVES * WAVE, 0, s>>>(
-            (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, gate, gate_ld, (bf16_t*)out, part, positions,
-            row_of_token, block_table, table_stride, page_size, n_tokens, heads, kv_heads, dim, vdim, n_pages, scale,
-            window, lambda, eps, out_scale, n_splits);
-        if (n_splits > 1) {
-            if (launch_status()) return IMPARO_LAUNCH_FAILED;
-            k_diff_merge<bf16_t><<<merge_blocks, DA_WAVES * WAVE, 0, s>>>(part, gate, gate_ld, (bf16_t*)out, positions,
-                                                                          n_tokens, heads, vdim, window, lambda, eps,
-                                                                          out_scale, n_splits);
-        }
-    } else {
-        return IMPARO_BAD_ARGUMENT;
-    }
+    if (dtype != IMPARO_F32 && dtype != IMPARO_BF16) return IMPARO_BAD_ARGUMENT;
+#define DA_LAUNCH(T, VPL)                                                                                              \
+    do {                                                                                                               \
+        k_diff_attention<T, VPL><<<(unsigned)blocks, DA_WAVES * WAVE, 0, s>>>(                                          \
+            (const T*)q, (const T*)k_cache, (const T*)v_cache, gate, gate_ld, (T*)out, part, positions, row_of_token,  \
+            block_table, table_stride, page_size, n_tokens, heads, kv_heads, dim, vdim, n_pages, scale, window, lambda, \
+            eps, out_scale, n_splits);                                                                                 \
+        if (n_splits > 1) {                                                                                            \
+            if (launch_status()) return IMPARO_LAUNCH_FAILED;                                                          \
+            k_diff_merge<T, VPL><<<merge_blocks, DA_WAVES * WAVE, 0, s>>>(part, gate, gate_ld, (T*)out, positions,      \
+                                                                         n_tokens, heads, vdim, window, lambda, eps,  \
+                                                                         out_scale, n_splits);                         \
+        }                                                                                                              \
+    } while (0)
+#define DA_LAUNCH_T(T)                  \
+    do {                                \
+        if (vdim <= 64) DA_LAUNCH(T, 1);       \
+        else if (vdim <= 128) DA_LAUNCH(T, 2); \
+        else if (vdim <= 256) DA_LAUNCH(T, 4); \
+        else DA_LAUNCH(T, 8);                  \
+    } while (0)
+    if (dtype == IMPARO_F32) DA_LAUNCH_T(float);
+    else DA_LAUNCH_T(bf16_t);
+#undef DA_LAUNCH_T
+#undef DA_LAUNCH
     return launch_status();
 }
 
 int imparo_load_code_diff_attention() {
     hipFuncAttributes attributes;
-    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_diff_attention<float>)) == hipSuccess
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_diff_attention<float, 1>)) == hipSuccess
                ? IMPARO_OK
                : IMPARO_LAUNCH_FAILED;
 }

@@ -125,58 +125,152 @@ extern "C" int imparo_causal_conv(const float* u, int u_ld, const float* weight,
 
 // ---------------------------------------------------------------- selective scan
 // A block takes 256 / LP channels of one request; LP lanes (a power of two, at most 64) share a
-// channel's states, SPL states a lane (n = lane + j * LP). The request's tokens are walked in order;
-// a token's contribution sum_n S[n] C[n] is added up across the LP lanes by a butterfly, the same
-// order whatever the batch.
-template <typename TX, typename TOut, int SPL>
+// channel's states, SPL states a lane (n = lane + j * LP). Tokens are walked in order, UNR at a time:
+// their inputs are asked for together, from clamped addresses, and a token past the end walks with a
+// step of zero, which leaves the state as it is. A token's sum_n S[n] C[n] is added up across the LP
+// lanes by a butterfly, the same order whatever the batch.
+//
+// A long segment is cut into chunks of SCAN_CHUNK tokens that run side by side: k_scan_chunk_state walks
+// every chunk but the last from a zero state and leaves its end state E_k and the sum of its steps (the
+// chunk's decay is exp(A sum dt)); k_selective_scan then starts chunk k from I_k, with I_0 the request's
+// state and I_{j+1} = exp(A sum_j) I_j + E_j, and walks it again, now with outputs. The request's state
+// is copied aside first (chunk 0 of the first launch), since the last chunk replaces it while others read.
+#define SCAN_CHUNK 64
+
+extern "C" int imparo_selective_scan_chunk(void) { return SCAN_CHUNK; }
+
+template <typename TX, typename TOut, int SPL, int UNR, bool EMIT>
+__device__ __forceinline__ float scan_walk(const float* __restrict__ dt_raw, const TX* __restrict__ x,
+                                           const float* __restrict__ bc, const float* __restrict__ z, int z_ld,
+                                           TOut* __restrict__ out, float (&S)[SPL], const float (&a)[SPL], float d_skip,
+                                           size_t t_first, int count, int channels, int cc, int n_state, int lp, int ln,
+                                           bool live) {
+    float dt_sum = 0.f;
+    for (int i = 0; i < count; i += UNR) {
+        float dt[UNR], xv[UNR], zv[UNR], b[UNR][SPL], cv[UNR][SPL];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            const size_t t = t_first + (size_t)min(i + u, count - 1);
+            dt[u] = dt_raw[t * channels + cc];
+            xv[u] = load_f32<TX>(x, t * channels + cc);
+            zv[u] = EMIT ? z[t * z_ld + cc] : 0.f;
+#pragma unroll
+            for (int j = 0; j < SPL; ++j) {
+                const int nn = min(ln + j * lp, n_state - 1);
+                b[u][j] = bc[t * 2 * n_state + nn];
+                cv[u][j] = EMIT ? bc[t * 2 * n_state + n_state + nn] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            const bool on = i + u < count;
+            const float step = on ? softplus_f32(dt[u]) : 0.f;
+            const float dx = step * xv[u];
+            dt_sum += step;
+            float y = 0.f;
+#pragma unroll
+            for (int j = 0; j < SPL; ++j) {
+                const bool has = ln + j * lp < n_state;
+                const float s_new = expf(step * a[j]) * S[j] + dx * b[u][j];
+                S[j] = has ? s_new : 0.f;
+                y += has ? s_new * cv[u][j] : 0.f;
+            }
+            if (EMIT) {
+                for (int off = lp >> 1; off > 0; off >>= 1) y += __shfl_xor(y, off, WAVE);
+                if (ln == 0 && live && on) {
+                    y += d_skip * xv[u];
+                    store_f32<TOut>(out, (t_first + i + u) * channels + cc, y * silu_f32(zv[u]));
+                }
+            }
+        }
+    }
+    return dt_sum;
+}
+
+// scratch: [rows, n_chunks, channels, n_state] end states, then [rows, n_chunks, channels] step sums, then
+// [rows, channels, n_state] the requests' states as they were.
+template <typename TX, int SPL, int UNR>
+__global__ void k_scan_chunk_state(const float* __restrict__ dt_raw, const TX* __restrict__ x,
+                                   const float* __restrict__ bc, const float* __restrict__ A,
+                                   const float* __restrict__ state, const int32_t* __restrict__ seg_start,
+                                   const int32_t* __restrict__ seg_len, const int32_t* __restrict__ slot,
+                                   float* __restrict__ scratch, int n_rows, int n_chunks, int channels, int n_state,
+                                   int lp) {
+    const int r = blockIdx.x, k = blockIdx.z;
+    const int len = seg_len[r];
+    const int chunks = (len + SCAN_CHUNK - 1) / SCAN_CHUNK;
+    if (chunks < 2 || k >= chunks - 1) return;
+    const int ln = threadIdx.x & (lp - 1);
+    const int c = blockIdx.y * (blockDim.x / lp) + threadIdx.x / lp;
+    const bool live = c < channels;
+    const int cc = live ? c : channels - 1;
+    float S[SPL], a[SPL];
+#pragma unroll
+    for (int j = 0; j < SPL; ++j) {
+        const int n = min(ln + j * lp, n_state - 1);
+        S[j] = 0.f;
+        a[j] = A[(size_t)cc * n_state + n];
+    }
+    const float sum = scan_walk<TX, float, SPL, UNR, false>(dt_raw, x, bc, nullptr, 0, nullptr, S, a, 0.f,
+                                                            (size_t)seg_start[r] + (size_t)k * SCAN_CHUNK, SCAN_CHUNK,
+                                                            channels, cc, n_state, lp, ln, live);
+    if (!live) return;
+    float* ends = scratch + (((size_t)r * n_chunks + k) * channels + cc) * n_state;
+    float* sums = scratch + (size_t)n_rows * n_chunks * channels * n_state + ((size_t)r * n_chunks + k) * channels;
+    float* was = scratch + (size_t)n_rows * n_chunks * channels * (n_state + 1) + ((size_t)r * channels + cc) * n_state;
+    const float* st = state + ((size_t)slot[r] * channels + cc) * n_state;
+#pragma unroll
+    for (int j = 0; j < SPL; ++j) {
+        const int n = ln + j * lp;
+        if (n < n_state) {
+            ends[n] = S[j];
+            if (k == 0) was[n] = st[n];
+        }
+    }
+    if (ln == 0) sums[cc] = sum;
+}
+
+template <typename TX, typename TOut, int SPL, int UNR>
 __global__ void k_selective_scan(const float* __restrict__ dt_raw, const TX* __restrict__ x,
                                  const float* __restrict__ bc, const float* __restrict__ z, int z_ld,
                                  const float* __restrict__ A, const float* __restrict__ D, float* __restrict__ state,
                                  const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len,
-                                 const int32_t* __restrict__ slot, TOut* __restrict__ out, int channels, int n_state,
+                                 const int32_t* __restrict__ slot, TOut* __restrict__ out,
+                                 const float* __restrict__ scratch, int n_rows, int n_chunks, int channels, int n_state,
                                  int lp) {
-    const int r = blockIdx.x;
+    const int r = blockIdx.x, k = blockIdx.z;
+    const int len = seg_len[r];
+    const int chunks = n_chunks > 1 ? max(1, (len + SCAN_CHUNK - 1) / SCAN_CHUNK) : 1;
+    if (k >= chunks) return;
     const int ln = threadIdx.x & (lp - 1);
     const int c = blockIdx.y * (blockDim.x / lp) + threadIdx.x / lp;
     const bool live = c < channels;
     const int cc = live ? c : channels - 1;            // lanes past the last channel repeat it and store nothing
     float S[SPL], a[SPL];
     float* st = state + ((size_t)slot[r] * channels + cc) * n_state;
+    const float* from = st;
+    if (chunks > 1)
+        from = scratch + (size_t)n_rows * n_chunks * channels * (n_state + 1) + ((size_t)r * channels + cc) * n_state;
 #pragma unroll
     for (int j = 0; j < SPL; ++j) {
-        const int n = ln + j * lp;
-        const bool on = n < n_state;
-        S[j] = on ? st[n] : 0.f;
-        a[j] = on ? A[(size_t)cc * n_state + n] : 0.f;
+        const int n = min(ln + j * lp, n_state - 1);
+        S[j] = ln + j * lp < n_state ? from[n] : 0.f;
+        a[j] = A[(size_t)cc * n_state + n];
     }
-    const float d_skip = D[cc];
-    const int t0 = seg_start[r];
-    const int len = seg_len[r];
-    for (int i = 0; i < len; ++i) {
-        const size_t t = (size_t)(t0 + i);
-        const float dt = softplus_f32(dt_raw[t * channels + cc]);
-        const float xv = load_f32<TX>(x, t * channels + cc);
-        const float dx = dt * xv;
-        float y = 0.f;
+    for (int p = 0; p < k; ++p) {                       // the chunks before this one, in order
+        const float* ends = scratch + (((size_t)r * n_chunks + p) * channels + cc) * n_state;
+        const float sum = scratch[(size_t)n_rows * n_chunks * channels * n_state + ((size_t)r * n_chunks + p) * channels + cc];
 #pragma unroll
         for (int j = 0; j < SPL; ++j) {
-            const int n = ln + j * lp;
-            const bool on = n < n_state;
-            const int nn = on ? n : 0;
-            const float b = bc[t * 2 * n_state + nn];
-            const float cv = bc[t * 2 * n_state + n_state + nn];
-            const float s_new = expf(dt * a[j]) * S[j] + dx * b;
-            S[j] = on ? s_new : 0.f;
-            y += on ? s_new * cv : 0.f;
-        }
-        for (int off = lp >> 1; off > 0; off >>= 1) y += __shfl_xor(y, off, WAVE);
-        if (ln == 0 && live) {
-            y += d_skip * xv;
-            const float zv = z[t * z_ld + cc];
-            store_f32<TOut>(out, t * channels + cc, y * silu_f32(zv));
+            const int n = min(ln + j * lp, n_state - 1);
+            S[j] = ln + j * lp < n_state ? expf(sum * a[j]) * S[j] + ends[n] : 0.f;
         }
     }
-    if (live) {
+    const int first = chunks > 1 ? k * SCAN_CHUNK : 0;
+    const int count = chunks > 1 ? min(SCAN_CHUNK, len - first) : len;
+    scan_walk<TX, TOut, SPL, UNR, true>(dt_raw, x, bc, z, z_ld, out, S, a, D[cc], (size_t)seg_start[r] + first, count,
+                                        channels, cc, n_state, lp, ln, live);
+    if (live && k == chunks - 1 && len > 0) {
 #pragma unroll
         for (int j = 0; j < SPL; ++j) {
             const int n = ln + j * lp;
@@ -188,21 +282,31 @@ __global__ void k_selective_scan(const float* __restrict__ dt_raw, const TX* __r
 template <typename TX, typename TOut>
 static int launch_scan(const float* dt_raw, const void* x, const float* bc, const float* z, int z_ld, const float* A,
                        const float* D, float* state, const int32_t* seg_start, const int32_t* seg_len,
-                       const int32_t* slot, void* out, int n_rows, int channels, int n_state, hipStream_t s) {
+                       const int32_t* slot, void* out, float* scratch, int n_chunks, int n_rows, int channels,
+                       int n_state, hipStream_t s) {
     int lp = 1;
     while (lp < n_state && lp < WAVE) lp <<= 1;
     const int spl = (n_state + lp - 1) / lp;
     const int threads = 256;
     const int per_block = threads / lp;
-    dim3 grid(n_rows, (channels + per_block - 1) / per_block);
-    if (grid.y > 65535) return IMPARO_BAD_ARGUMENT;
-#define SCAN_LAUNCH(N) \
-    k_selective_scan<TX, TOut, N><<<grid, threads, 0, s>>>(dt_raw, (const TX*)x, bc, z, z_ld, A, D, state, seg_start, \
-                                                           seg_len, slot, (TOut*)out, channels, n_state, lp)
-    if (spl == 1) SCAN_LAUNCH(1);
-    else if (spl == 2) SCAN_LAUNCH(2);
-    else if (spl <= 4) SCAN_LAUNCH(4);
-    else if (spl <= 8) SCAN_LAUNCH(8);
+    dim3 grid(n_rows, (channels + per_block - 1) / per_block, n_chunks);
+    if (grid.y > 65535 || grid.z > 65535) return IMPARO_BAD_ARGUMENT;
+#define SCAN_LAUNCH(N, U)                                                                                             \
+    do {                                                                                                              \
+        if (n_chunks > 1) {                                                                                           \
+            k_scan_chunk_state<TX, N, U><<<grid, threads, 0, s>>>(dt_raw, (const TX*)x, bc, A, state, seg_start,      \
+                                                                  seg_len, slot, scratch, n_rows, n_chunks, channels, \
+                                                                  n_state, lp);                                       \
+            if (launch_status()) return IMPARO_LAUNCH_FAILED;                                                         \
+        }                                                                                                             \
+        k_selective_scan<TX, TOut, N, U><<<grid, threads, 0, s>>>(dt_raw, (const TX*)x, bc, z, z_ld, A, D, state,     \
+                                                                  seg_start, seg_len, slot, (TOut*)out, scratch,      \
+                                                                  n_rows, n_chunks, channels, n_state, lp);           \
+    } while (0)
+    if (spl == 1) SCAN_LAUNCH(1, 8);
+    else if (spl == 2) SCAN_LAUNCH(2, 4);
+    else if (spl <= 4) SCAN_LAUNCH(4, 2);
+    else if (spl <= 8) SCAN_LAUNCH(8, 1);
     else return IMPARO_BAD_ARGUMENT;
 #undef SCAN_LAUNCH
     return launch_status();
@@ -211,22 +315,25 @@ static int launch_scan(const float* dt_raw, const void* x, const float* bc, cons
 // dt_raw [tokens, channels] float32 (the step projection with its bias, before softplus); x [tokens,
 // channels] in `dtype`; bc [tokens, 2 n_state] float32 (B then C); z rows z_ld floats apart; A, D float32
 // (A = -exp(A_log), [channels, n_state]); state [slots, channels, n_state] float32; out [tokens, channels]
-// in `dtype`. n_state at most 512.
+// in `dtype`. n_state at most 512. n_chunks 1: every segment is walked in one piece. More (at least
+// ceil(longest segment / imparo_selective_scan_chunk())): segments are walked in chunks side by side through
+// `scratch`, n_rows * (n_chunks * channels * (n_state + 1) + channels * n_state) floats.
 extern "C" int imparo_selective_scan(const float* dt_raw, const void* x, const float* bc, const float* z, int z_ld,
                                      const float* A, const float* D, float* state, const int32_t* seg_start,
-                                     const int32_t* seg_len, const int32_t* slot, void* out, int dtype, int n_rows,
-                                     int channels, int n_state, imparo_stream stream) {
+                                     const int32_t* seg_len, const int32_t* slot, void* out, int dtype, float* scratch,
+                                     int n_chunks, int n_rows, int channels, int n_state, imparo_stream stream) {
     if (!dt_raw || !x || !bc || !z || !A || !D || !state || !seg_start || !seg_len || !slot || !out)
         return IMPARO_BAD_ARGUMENT;
     if (n_rows < 0 || channels <= 0 || n_state <= 0 || n_state > 512 || z_ld < channels) return IMPARO_BAD_ARGUMENT;
+    if (n_chunks < 1 || (n_chunks > 1 && !scratch)) return IMPARO_BAD_ARGUMENT;
     if (n_rows == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == IMPARO_F32)
-        return launch_scan<float, float>(dt_raw, x, bc, z, z_ld, A, D, state, seg_start, seg_len, slot, out, n_rows,
-                                         channels, n_state, s);
+        return launch_scan<float, float>(dt_raw, x, bc, z, z_ld, A, D, state, seg_start, seg_len, slot, out, scratch,
+                                         n_chunks, n_rows, channels, n_state, s);
     if (dtype == IMPARO_BF16)
-        return launch_scan<bf16_t, bf16_t>(dt_raw, x, bc, z, z_ld, A, D, state, seg_start, seg_len, slot, out, n_rows,
-                                           channels, n_state, s);
+        return launch_scan<bf16_t, bf16_t>(dt_raw, x, bc, z, z_ld, A, D, state, seg_start, seg_len, slot, out, scratch,
+                                           n_chunks, n_rows, channels, n_state, s);
     return IMPARO_BAD_ARGUMENT;
 }
 

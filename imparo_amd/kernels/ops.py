@@ -612,23 +612,39 @@ def causal_conv(u: torch.Tensor, channels: int, weight: torch.Tensor, bias: Opti
     return out
 
 
+def selective_scan_chunk() -> int:
+    """Tokens per chunk when `selective_scan` walks long segments in chunks side by side."""
+    return int(library().imparo_selective_scan_chunk())
+
+
+def selective_scan_scratch(n_rows: int, n_chunks: int, channels: int, n_state: int) -> int:
+    """Floats of scratch that `selective_scan` needs for `n_chunks` > 1."""
+    return n_rows * (n_chunks * channels * (n_state + 1) + channels * n_state)
+
+
 def selective_scan(dt_raw: torch.Tensor, x: torch.Tensor, bc: torch.Tensor, z: torch.Tensor, z_ld: int, A: torch.Tensor,
                    D: torch.Tensor, state: torch.Tensor, seg_start: torch.Tensor, seg_len: torch.Tensor,
-                   slot: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+                   slot: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tensor] = None,
+                   n_chunks: int = 1) -> torch.Tensor:
     """The selective scan of every request's segment, continued from its state [slots, channels, n_state]
     (float32), which is advanced. dt_raw [tokens, channels] float32 before softplus; x and out [tokens,
-    channels] in one dtype; bc [tokens, 2 n_state] float32; z a float32 view whose rows lie z_ld apart."""
+    channels] in one dtype; bc [tokens, 2 n_state] float32; z a float32 view whose rows lie z_ld apart.
+    `n_chunks` > 1 (at least ceil(longest segment / selective_scan_chunk())): the chunks of a segment run
+    side by side through `scratch` (selective_scan_scratch floats); the caller knows the longest segment."""
     n, channels = x.shape
     n_state = A.shape[1]
     n_rows = seg_start.shape[0]
     if z.dtype != torch.float32 or z.device != x.device or z_ld < channels:
         raise KernelArgumentError("selective_scan: z is float32 on the GPU, its rows at least `channels` apart")
+    if n_chunks > 1 and (scratch is None or scratch.numel() < selective_scan_scratch(n_rows, n_chunks, channels, n_state)):
+        raise KernelArgumentError("selective_scan: the scratch for the chunks' states is too small")
     _check(library().imparo_selective_scan(
         _dev(dt_raw, "dt", torch.float32, (n, channels)), _dev(x, "scan x"), _dev(bc, "B and C", torch.float32, (n, 2 * n_state)),
         z.data_ptr(), int(z_ld), _dev(A, "A", torch.float32, (channels, n_state)), _dev(D, "D", torch.float32, (channels,)),
         _dev(state, "scan state", torch.float32, (state.shape[0], channels, n_state)),
         _dev(seg_start, "seg_start", torch.int32, (n_rows,)), _dev(seg_len, "seg_len", torch.int32, (n_rows,)),
         _dev(slot, "slot", torch.int32, (n_rows,)), _dev(out, "scan out", x.dtype, (n, channels)), _code(x, "scan x"),
+        _dev(scratch, "scan scratch", torch.float32) if n_chunks > 1 else 0, int(n_chunks),
         n_rows, channels, n_state, _stream()), "selective_scan")
     return out
 

@@ -109,8 +109,15 @@ class SelectiveScan:
         y = ctx.workspace.get("scan_y", (T, self.inner), self.out_proj.in_dtype, alias="mixer_mid")
         if y.dtype != x.dtype:
             raise ValueError("the scan's input and output projections differ in dtype")
+        # a long portion is walked in chunks side by side (their end states meet in scratch)
+        chunk = ops.selective_scan_chunk()
+        n_chunks = -(-ctx.max_seg_len // chunk) if ctx.max_seg_len > chunk + chunk // 2 else 1
+        scratch = None
+        if n_chunks > 1:
+            scratch = ctx.workspace.get("scan_chunks", (ops.selective_scan_scratch(ctx.n_rows, n_chunks, self.inner,
+                                                                                   self.n_state),), torch.float32)
         ops.selective_scan(dt, x, bc, xz[:, self.inner:], 2 * self.inner, self.A, self.D, state["scan"],
-                           ctx.seg_start, ctx.seg_len, ctx.slot, y)
+                           ctx.seg_start, ctx.seg_len, ctx.slot, y, scratch, n_chunks)
         return self.out_proj(ctx, y, torch.float32, "mixer_out", sliced_ok=True, into=ctx.stream)
 
 

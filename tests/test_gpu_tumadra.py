@@ -171,25 +171,61 @@ def test_causal_conv_kernel_continues(taps):
 @pytest.mark.parametrize("C,N", [(24, 8), (40, 20), (16, 1), (8, 80)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_selective_scan_kernel_continues(C, N, dtype):
+    """One sequence in segments of 1 to 200 tokens, the long ones walked in chunks side by side: the state
+    carries from segment to segment and from chunk to chunk; other slots stay untouched."""
     from imparo_amd.kernels import ops
     g = torch.Generator().manual_seed(C * N)
-    T = 23
+    cuts = (1, 7, 2, 1, 12, 200, 97, 130)
+    T = sum(cuts)
     dt_raw, x = torch.randn(T, C, generator=g) - 2, torch.randn(T, C, generator=g).to(dtype).float()
     bc, z = torch.randn(T, 2 * N, generator=g), torch.randn(T, 2 * C, generator=g)
     A, D = -torch.rand(C, N, generator=g) * 6, torch.randn(C, generator=g)
     ref = plain.scan(torch.nn.functional.softplus(dt_raw), x, bc[:, :N], bc[:, N:], A, D) * torch.nn.functional.silu(z[:, C:])
     state = dev(torch.zeros(5, C, N))
+    chunk = ops.selective_scan_chunk()
     got, at = [], 0
-    for n in (1, 7, 2, 1, 12):
+    for n in cuts:
         out = torch.empty(n, C, device=DEV, dtype=dtype)
         zz = dev(z[at:at + n])
+        n_chunks = -(-n // chunk) if n > chunk + chunk // 2 else 1
+        scratch = torch.full((ops.selective_scan_scratch(1, n_chunks, C, N),), float("nan"), device=DEV) if n_chunks > 1 else None
         ops.selective_scan(dev(dt_raw[at:at + n]), dev(x[at:at + n], dtype), dev(bc[at:at + n]), zz[:, C:], 2 * C, dev(A),
-                           dev(D), state, i32([0]), i32([n]), i32([3]), out)
+                           dev(D), state, i32([0]), i32([n]), i32([3]), out, scratch, n_chunks)
         got.append(out.float().cpu())
         at += n
     tol = 1e-5 if dtype == torch.float32 else 2e-2
     assert torch.allclose(torch.cat(got), ref, atol=tol * float(ref.abs().max()), rtol=tol)
     assert float(state[[0, 1, 2, 4]].abs().max()) == 0.0
+
+
+def test_selective_scan_kernel_rows_of_unequal_length():
+    """Three requests in one launch, 150, 1 and 70 tokens: chunks for the long one only; each equals its own run."""
+    from imparo_amd.kernels import ops
+    g = torch.Generator().manual_seed(77)
+    C, N, lens = 24, 12, [150, 1, 70]
+    T = sum(lens)
+    dt_raw, x = torch.randn(T, C, generator=g) - 2, torch.randn(T, C, generator=g)
+    bc, z = torch.randn(T, 2 * N, generator=g), torch.randn(T, 2 * C, generator=g)
+    A, D = -torch.rand(C, N, generator=g) * 6, torch.randn(C, generator=g)
+    first = torch.randn(4, C, N, generator=g)
+    state = dev(first)
+    out = torch.empty(T, C, device=DEV)
+    chunk = ops.selective_scan_chunk()
+    n_chunks = -(-max(lens) // chunk)
+    scratch = torch.full((ops.selective_scan_scratch(3, n_chunks, C, N),), float("nan"), device=DEV)
+    zz = dev(z)
+    ops.selective_scan(dev(dt_raw), dev(x), dev(bc), zz[:, C:], 2 * C, dev(A), dev(D), state, i32([0, 150, 151]),
+                       i32(lens), i32([2, 0, 3]), out, scratch, n_chunks)
+    at = 0
+    for n, s in zip(lens, [2, 0, 3]):
+        S = first[s].clone()
+        sl = slice(at, at + n)
+        ref = plain.scan(torch.nn.functional.softplus(dt_raw[sl]), x[sl], bc[sl, :N], bc[sl, N:], A, D, S) \
+            * torch.nn.functional.silu(z[sl, C:])
+        assert torch.allclose(out[sl].cpu(), ref, atol=2e-5 * float(ref.abs().max()), rtol=2e-5)
+        assert torch.allclose(state[s].cpu(), S, atol=1e-5, rtol=1e-5)
+        at += n
+    assert torch.equal(state[1].cpu(), first[1])
 
 
 def attention_case(H, G, D, V, n_ctx, page, dtype, far=None, seed=0):
