@@ -268,11 +268,24 @@ int imparo_diff_qkv_store(const float* rows_in, int ld, const int32_t* positions
 // out = o / sqrt(mean(o^2) + eps) * out_scale * sigmoid(gate) (gate null: no gate). n_splits > 1 walks the
 // keys in pieces of imparo_diff_attention_split() through `part` (tokens x heads x n_splits x (2 vdim + 4) floats).
 int imparo_diff_attention_split(void);
+// below > 0: only the tokens of rows (seg_len per row) that bring fewer than `below` tokens.
 int imparo_diff_attention(const void* q, const void* k_cache, const void* v_cache, const float* gate, int gate_ld,
                           void* out, float* part, int dtype, const int32_t* positions, const int32_t* row_of_token,
                           const int32_t* block_table, int table_stride, int page_size, int n_tokens, int heads,
                           int kv_heads, int dim, int vdim, int n_pages, float scale, int window, float lambda,
-                          float eps, float out_scale, int n_splits, imparo_stream stream);
+                          float eps, float out_scale, int n_splits, const int32_t* seg_len, int below,
+                          imparo_stream stream);
+// The same on the matrix cores, for rows that bring portions: bfloat16, pages of a multiple of 16 positions, dim
+// and vdim multiples of 4 up to 128 (imparo_diff_attention_tiles_takes). A block takes
+// imparo_diff_attention_tile() queries of one row and one head; rows of fewer than min_len tokens are skipped.
+int imparo_diff_attention_tile(void);
+int imparo_diff_attention_tiles_takes(int page_size, int dim, int vdim);
+int imparo_diff_attention_tiles(const void* q, const void* k_cache, const void* v_cache, const float* gate,
+                                int gate_ld, void* out, const int32_t* positions, const int32_t* seg_start,
+                                const int32_t* seg_len, const int32_t* block_table, int table_stride, int page_size,
+                                int n_rows, int max_seg_len, int heads, int kv_heads, int dim, int vdim, int n_pages,
+                                float scale, int window, float lambda, float eps, float out_scale, int min_len,
+                                imparo_stream stream);
 
 // ---------------------------------------------------------------------------------------------
 // A model's step as one call. A program is the model's run order as a list of operations over a

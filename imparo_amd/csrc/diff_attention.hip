@@ -124,7 +124,7 @@ __global__ void k_diff_attention(const T* __restrict__ q, const T* __restrict__ 
                                  const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ block_table,
                                  int table_stride, int page_size, int n_tokens, int heads, int kv_heads, int dim,
                                  int vdim, int n_pages, float scale, int window, float lambda, float eps,
-                                 float out_scale, int n_splits) {
+                                 float out_scale, int n_splits, const int32_t* __restrict__ seg_len, int below) {
     __shared__ float q_rows[DA_WAVES][2 * DA_MAX_DIM];
     __shared__ float probs[DA_WAVES][2][WAVE];
     __shared__ long long v_off[DA_WAVES][WAVE];
@@ -137,6 +137,7 @@ __global__ void k_diff_attention(const T* __restrict__ q, const T* __restrict__ 
     const int t = (int)(th / heads);
     const int h = (int)(th - (long long)t * heads);
     const int g = h / (heads / kv_heads);
+    if (below > 0 && seg_len[row_of_token[t]] >= below) return;   // a longer row's tokens are another launch's
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
     int first = (lo / WAVE) * WAVE, last = pos;             // chunks from `first`, keys up to `last`
@@ -253,11 +254,13 @@ __global__ void k_diff_attention(const T* __restrict__ q, const T* __restrict__ 
 template <typename T, int VPL>
 __global__ void k_diff_merge(const float* __restrict__ part, const float* __restrict__ gate, int gate_ld,
                              T* __restrict__ out, const int32_t* __restrict__ positions, int n_tokens, int heads,
-                             int vdim, int window, float lambda, float eps, float out_scale, int n_splits) {
+                             int vdim, int window, float lambda, float eps, float out_scale, int n_splits,
+                             const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ seg_len, int below) {
     const int lane = threadIdx.x & (WAVE - 1);
     const long long th = (long long)blockIdx.x * DA_WAVES + threadIdx.x / WAVE;
     if (th >= (long long)n_tokens * heads) return;
     const int t = (int)(th / heads);
+    if (below > 0 && seg_len[row_of_token[t]] >= below) return;
     const int h = (int)(th - (long long)t * heads);
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
@@ -298,6 +301,236 @@ __global__ void k_diff_merge(const float* __restrict__ part, const float* __rest
                  out + ((size_t)t * heads + h) * vdim, vdim, lane);
 }
 
+// ---------------------------------------------------------------- matrix-core kernel for prompt portions
+// bfloat16, pages of a multiple of 16 positions, dim and vdim multiples of 4 up to 128. A block is four
+// waves of one head over 64 consecutive queries of one request's portion, a wave takes 16 of them. Keys
+// are walked in tiles of 32 at absolute multiples of 32. Both products are taken transposed, S^T = K Q^T
+// and O^T = V^T P^T (16x16x16 products): the scores a lane holds after the first product (four
+// consecutive keys of one query) are exactly what the second wants from it as its right operand, so no
+// value crosses lanes between the two; a query's maximum and sum meet over the four lanes that share its
+// column. Each map keeps its own maximum, sum and O^T; both share every V^T operand.
+typedef short da_s16x4 __attribute__((ext_vector_type(4)));
+typedef float da_f32x4 __attribute__((ext_vector_type(4)));
+#define DAM_TILE 64          // queries a block
+#define DAM_MAX16 8          // 16-wide blocks of dim and of vdim that the registers hold
+
+extern "C" int imparo_diff_attention_tile(void) { return DAM_TILE; }
+
+__device__ __forceinline__ da_s16x4 da_pack4(float a, float b, float c, float d) {
+    const uint32_t lo = f32x2_to_bf16x2(a, b), hi = f32x2_to_bf16x2(c, d);
+    da_s16x4 r;
+    r[0] = (short)(lo & 0xffff);
+    r[1] = (short)(lo >> 16);
+    r[2] = (short)(hi & 0xffff);
+    r[3] = (short)(hi >> 16);
+    return r;
+}
+
+__global__ __launch_bounds__(256) void k_diff_attention_tiles(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const float* __restrict__ gate, int gate_ld, bf16_t* __restrict__ out, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len,
+    const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int dim,
+    int vdim, int n_pages, float scale, int window, float lambda, float eps, float out_scale, int min_len) {
+    const int r = blockIdx.x, h = blockIdx.z;
+    const int len = seg_len[r];
+    if (len < min_len) return;                                 // (uniform over the block) such rows are another launch's
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int q0 = blockIdx.y * DAM_TILE + wave * 16;          // this wave's first query within the portion
+    if (q0 >= len) return;
+    const int col = lane & 15, quad = lane >> 4;               // a lane's query column and its group of four rows
+    const int t0 = seg_start[r];
+    const int n_q = min(16, len - q0);
+    const int qi = min(col, n_q - 1);                          // columns past the portion repeat its last query and store nothing
+    const int t = t0 + q0 + qi;
+    const int pos = positions[t];
+    const int pos_first = positions[t0 + q0], pos_last = positions[t0 + q0 + n_q - 1];
+    const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    const int lo_first = window > 0 ? max(0, pos_first + 1 - window) : 0;
+    const int g = h / (heads / kv_heads);
+    const int dim16 = (dim + 15) >> 4, vd16 = (vdim + 15) >> 4;
+    const int32_t* table = block_table + (size_t)r * table_stride;
+
+    // Q^T operands: query `col`, dims 16 kk + 4 quad .. + 3, both maps
+    da_s16x4 qf[2][DAM_MAX16];
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int kk = 0; kk < DAM_MAX16; ++kk) {
+            const int d = kk * 16 + quad * 4;
+            const bool on = kk < dim16 && d < dim;
+            const bf16_t* src = q + (((size_t)t * heads + h) * 2 + m) * dim + (on ? d : 0);
+            const da_s16x4 v = *reinterpret_cast<const da_s16x4*>(src);
+            qf[m][kk] = on ? v : da_s16x4{0, 0, 0, 0};
+        }
+    da_f32x4 o[2][DAM_MAX16];
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int vb = 0; vb < DAM_MAX16; ++vb) o[m][vb] = da_f32x4{0.f, 0.f, 0.f, 0.f};
+    float mx[2] = {-INFINITY, -INFINITY}, sum[2] = {0.f, 0.f};
+
+    for (int k0 = (lo_first / 32) * 32; k0 <= pos_last; k0 += 32) {
+        // the two blocks of 16 keys of this tile lie in one page each
+        long long kbase[2], vbase[2];
+        bool there[2];
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+            const int key0 = k0 + mb * 16;
+            const int page = key0 <= pos_last ? table[key0 / page_size] : -1;
+            there[mb] = page >= 0 && page < n_pages;
+            const long long pg = there[mb] ? page : 0;
+            kbase[mb] = ((pg * 2 * kv_heads + 2 * g) * page_size + (key0 % page_size)) * dim;
+            vbase[mb] = ((pg * kv_heads + g) * page_size + (key0 % page_size)) * (long long)vdim;
+        }
+        da_s16x4 pb[2][2];                                   // P^T operands: [map][block of 16 keys]
+        float corr[2];
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            da_f32x4 sc[2] = {da_f32x4{0.f, 0.f, 0.f, 0.f}, da_f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int kk = 0; kk < DAM_MAX16; ++kk) {
+                    if (kk < dim16) {
+                        const int d = kk * 16 + quad * 4;
+                        const bool on = d < dim;
+                        // key row `col` of the block, map m, dims d .. d + 3
+                        const bf16_t* src = k_cache + kbase[mb] + ((long long)m * page_size + col) * dim + (on ? d : 0);
+                        const da_s16x4 kv = *reinterpret_cast<const da_s16x4*>(src);
+                        sc[mb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(on ? kv : da_s16x4{0, 0, 0, 0}, qf[m][kk], sc[mb], 0, 0, 0);
+                    }
+                }
+            // a lane holds keys k0 + 16 mb + 4 quad + i of query `col`
+            float tile_max = -INFINITY;
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = k0 + mb * 16 + quad * 4 + i;
+                    const bool seen = there[mb] && key <= pos && key >= lo;
+                    sc[mb][i] = seen ? sc[mb][i] * scale : -INFINITY;
+                    tile_max = fmaxf(tile_max, sc[mb][i]);
+                }
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
+            const float m_new = fmaxf(mx[m], tile_max);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            corr[m] = mx[m] == -INFINITY ? 0.f : __expf(mx[m] - m_use);
+            float tile_sum = 0.f;
+            float p[2][4];
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    p[mb][i] = __expf(sc[mb][i] - m_use);       // exp(-inf) = 0 for keys that are not seen
+                    tile_sum += p[mb][i];
+                }
+            tile_sum += __shfl_xor(tile_sum, 16, WAVE);
+            tile_sum += __shfl_xor(tile_sum, 32, WAVE);
+            sum[m] = sum[m] * corr[m] + tile_sum;
+            mx[m] = m_new;
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) pb[m][mb] = da_pack4(p[mb][0], p[mb][1], p[mb][2], p[mb][3]);
+        }
+#pragma unroll
+        for (int vb = 0; vb < DAM_MAX16; ++vb) {
+            if (vb < vd16) {
+#pragma unroll
+                for (int m = 0; m < 2; ++m) {
+                    o[m][vb][0] *= corr[m];
+                    o[m][vb][1] *= corr[m];
+                    o[m][vb][2] *= corr[m];
+                    o[m][vb][3] *= corr[m];
+                }
+                const int d = vb * 16 + col;                   // V^T row of this lane
+                const bool on_d = d < vdim;
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb) {
+                    // keys 4 quad .. + 3 of the block, value dimension d: four rows of V, one value each
+                    const bf16_t* src = v_cache + vbase[mb] + (long long)(quad * 4) * vdim + (on_d ? d : 0);
+                    da_s16x4 vt;
+                    vt[0] = (short)src[0];
+                    vt[1] = (short)src[vdim];
+                    vt[2] = (short)src[2 * vdim];
+                    vt[3] = (short)src[3 * vdim];
+                    const int key = k0 + mb * 16 + quad * 4;         // what lies past the last query's position is not a value yet
+                    if (key + 1 > pos_last) vt[1] = 0;
+                    if (key + 2 > pos_last) vt[2] = 0;
+                    if (key + 3 > pos_last) vt[3] = 0;
+                    if (!(on_d && there[mb]) || key > pos_last) vt = da_s16x4{0, 0, 0, 0};
+                    o[0][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt, pb[0][mb], o[0][vb], 0, 0, 0);
+                    o[1][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt, pb[1][mb], o[1][vb], 0, 0, 0);
+                }
+            }
+        }
+    }
+    // finish: a lane holds value dimensions 16 vb + 4 quad + i of query `col`
+    const float i1 = sum[0] > 0.f ? 1.0f / sum[0] : 0.f, i2 = sum[1] > 0.f ? 1.0f / sum[1] : 0.f;
+    float ss = 0.f;
+#pragma unroll
+    for (int vb = 0; vb < DAM_MAX16; ++vb)
+        if (vb < vd16) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool on = vb * 16 + quad * 4 + i < vdim;
+                const float v = on ? o[0][vb][i] * i1 - lambda * (o[1][vb][i] * i2) : 0.f;
+                o[0][vb][i] = v;
+                ss += v * v;
+            }
+        }
+    ss += __shfl_xor(ss, 16, WAVE);
+    ss += __shfl_xor(ss, 32, WAVE);
+    const float rr = out_scale / sqrtf(ss / (float)vdim + eps);
+    if (col < n_q) {
+        const float* gt = gate ? gate + (size_t)t * gate_ld + (size_t)h * vdim : nullptr;
+        bf16_t* dst = out + ((size_t)t * heads + h) * vdim;
+#pragma unroll
+        for (int vb = 0; vb < DAM_MAX16; ++vb)
+            if (vb < vd16) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int d = vb * 16 + quad * 4 + i;
+                    if (d < vdim) {
+                        float y = o[0][vb][i] * rr;
+                        if (gt) y *= 1.0f / (1.0f + __expf(-gt[d]));
+                        dst[d] = f32_to_bf16(y);
+                    }
+                }
+            }
+    }
+}
+
+// Whether the matrix-core kernel takes these sizes (bfloat16 only).
+extern "C" int imparo_diff_attention_tiles_takes(int page_size, int dim, int vdim) {
+    return page_size >= 16 && page_size % 16 == 0 && dim > 0 && vdim > 0 && dim % 4 == 0 && vdim % 4 == 0 &&
+           dim <= 16 * DAM_MAX16 && vdim <= 16 * DAM_MAX16;
+}
+
+// Differential attention of whole portions: every token of every row (seg_start, seg_len) of at least min_len
+// tokens, a row's tokens at consecutive positions. max_seg_len bounds every row's tokens. Sizes as imparo_diff_attention_tiles_takes says.
+extern "C" int imparo_diff_attention_tiles(const void* q, const void* k_cache, const void* v_cache, const float* gate,
+                                           int gate_ld, void* out, const int32_t* positions, const int32_t* seg_start,
+                                           const int32_t* seg_len, const int32_t* block_table, int table_stride,
+                                           int page_size, int n_rows, int max_seg_len, int heads, int kv_heads, int dim,
+                                           int vdim, int n_pages, float scale, int window, float lambda, float eps,
+                                           float out_scale, int min_len, imparo_stream stream) {
+    if (!q || !k_cache || !v_cache || !out || !positions || !seg_start || !seg_len || !block_table) return IMPARO_BAD_ARGUMENT;
+    if (n_rows < 0 || max_seg_len < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads) return IMPARO_BAD_ARGUMENT;
+    if (!imparo_diff_attention_tiles_takes(page_size, dim, vdim)) return IMPARO_BAD_ARGUMENT;
+    if (table_stride <= 0 || n_pages <= 0 || window < 0 || heads > 65535) return IMPARO_BAD_ARGUMENT;
+    if (gate && gate_ld < heads * vdim) return IMPARO_BAD_ARGUMENT;
+    if (n_rows == 0 || max_seg_len == 0) return IMPARO_OK;
+    const int tiles = (max_seg_len + DAM_TILE - 1) / DAM_TILE;
+    if (tiles > 65535) return IMPARO_BAD_ARGUMENT;
+    dim3 grid(n_rows, tiles, heads);
+    k_diff_attention_tiles<<<grid, 256, 0, (hipStream_t)stream>>>(
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, gate, gate_ld, (bf16_t*)out, positions, seg_start,
+        seg_len, block_table, table_stride, page_size, heads, kv_heads, dim, vdim, n_pages, scale, window, lambda, eps,
+        out_scale, min_len);
+    return launch_status();
+}
+
 extern "C" int imparo_diff_qkv_store(const float* rows_in, int ld, const int32_t* positions, const int32_t* row_of_token,
                                      const int32_t* block_table, int table_stride, int page_size, void* q_out,
                                      void* k_cache, void* v_cache, int dtype, int write_kv, int n_tokens, int heads,
@@ -326,13 +559,16 @@ extern "C" int imparo_diff_qkv_store(const float* rows_in, int ld, const int32_t
 // q [tokens, heads, 2, dim]; gate (may be null) float32 rows gate_ld apart, heads * vdim values a row, the
 // gate's logits; out [tokens, heads * vdim]. n_splits 1: no partial results; more: part holds
 // tokens * heads * n_splits * (2 vdim + 4) floats and n_splits covers every key (ceil(longest context / split)).
+// below > 0: only the tokens of rows that bring fewer than `below` tokens (seg_len per row); the others' outputs
+// are left as they are.
 extern "C" int imparo_diff_attention(const void* q, const void* k_cache, const void* v_cache, const float* gate,
                                      int gate_ld, void* out, float* part, int dtype, const int32_t* positions,
                                      const int32_t* row_of_token, const int32_t* block_table, int table_stride,
                                      int page_size, int n_tokens, int heads, int kv_heads, int dim, int vdim,
                                      int n_pages, float scale, int window, float lambda, float eps, float out_scale,
-                                     int n_splits, imparo_stream stream) {
+                                     int n_splits, const int32_t* seg_len, int below, imparo_stream stream) {
     if (!q || !k_cache || !v_cache || !out || !positions || !row_of_token || !block_table) return IMPARO_BAD_ARGUMENT;
+    if (below < 0 || (below > 0 && !seg_len)) return IMPARO_BAD_ARGUMENT;
     if (n_tokens < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads) return IMPARO_BAD_ARGUMENT;
     if (dim <= 0 || dim > DA_MAX_DIM || vdim <= 0 || vdim > DA_MAX_VDIM) return IMPARO_BAD_ARGUMENT;
     if (page_size <= 0 || table_stride <= 0 || n_pages <= 0 || window < 0 || n_splits < 1) return IMPARO_BAD_ARGUMENT;
@@ -350,12 +586,13 @@ extern "C" int imparo_diff_attention(const void* q, const void* k_cache, const v
         k_diff_attention<T, VPL><<<(unsigned)blocks, DA_WAVES * WAVE, 0, s>>>(                                          \
             (const T*)q, (const T*)k_cache, (const T*)v_cache, gate, gate_ld, (T*)out, part, positions, row_of_token,  \
             block_table, table_stride, page_size, n_tokens, heads, kv_heads, dim, vdim, n_pages, scale, window, lambda, \
-            eps, out_scale, n_splits);                                                                                 \
+            eps, out_scale, n_splits, seg_len, below);                                                                 \
         if (n_splits > 1) {                                                                                            \
             if (launch_status()) return IMPARO_LAUNCH_FAILED;                                                          \
             k_diff_merge<T, VPL><<<merge_blocks, DA_WAVES * WAVE, 0, s>>>(part, gate, gate_ld, (T*)out, positions,      \
                                                                          n_tokens, heads, vdim, window, lambda, eps,  \
-                                                                         out_scale, n_splits);                         \
+                                                                         out_scale, n_splits, row_of_token, seg_len,   \
+                                                                         below);                                       \
         }                                                                                                              \
     } while (0)
 #define DA_LAUNCH_T(T)                  \

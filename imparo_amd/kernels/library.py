@@ -61,7 +61,10 @@ _SIGNATURES = {
     "imparo_diff_attention_split": [],
     # q, k_cache, v_cache, gate, gate_ld, out, part, dtype, positions, row_of_token, table, stride, page, tokens, heads,
     # kv_heads, dim, vdim, n_pages, scale, window, lambda, eps, out_scale, n_splits, stream
-    "imparo_diff_attention": [P, P, P, P, I, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, F, F, F, I, P],
+    "imparo_diff_attention": [P, P, P, P, I, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, F, F, F, I, P, I, P],
+    "imparo_diff_attention_tile": [],
+    "imparo_diff_attention_tiles_takes": [I, I, I],
+    "imparo_diff_attention_tiles": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, I, F, F, F, I, P],
     "imparo_rows_parts": [I],
     # x, ssq_in, n_parts, eps, w, bias, y, out_dtype, x_io, ssq_out, weighted_out, weighted_by, m, n, k, epilogue, stream
     "imparo_rows_gemm": [P, P, I, F, P, P, P, I, P, P, P, P, I, I, I, I, P],

@@ -683,8 +683,10 @@ def diff_qkv_store(rows_in: torch.Tensor, positions: torch.Tensor, row_of_token:
 def diff_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gate: Optional[torch.Tensor],
                    gate_ld: int, out: torch.Tensor, positions: torch.Tensor, row_of_token: torch.Tensor,
                    block_table: torch.Tensor, scale: float, window: Optional[int], lam: float, eps: float,
-                   out_scale: float, part: Optional[torch.Tensor] = None, n_splits: int = 1) -> torch.Tensor:
-    """Differential attention of every token over its request's cached keys (see imparo_diff_attention)."""
+                   out_scale: float, part: Optional[torch.Tensor] = None, n_splits: int = 1,
+                   seg_len: Optional[torch.Tensor] = None, below: int = 0) -> torch.Tensor:
+    """Differential attention of every token over its request's cached keys (see imparo_diff_attention).
+    `below` > 0: only the tokens of rows that bring fewer than that many tokens (`seg_len` per row)."""
     n, heads, two, dim = q.shape
     n_pages, kv2, page_size, kdim = k_cache.shape
     kv_heads, vdim = v_cache.shape[1], v_cache.shape[3]
@@ -700,6 +702,39 @@ def diff_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         int(gate_ld), _dev(out, "attention out", q.dtype, (n, heads * vdim)), _dev(part, "partial results", torch.float32),
         _code(q, "q"), _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
         _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size, n, heads, kv_heads, dim, vdim,
-        n_pages, float(scale), int(window or 0), float(lam), float(eps), float(out_scale), int(n_splits), _stream()),
-        "diff_attention")
+        n_pages, float(scale), int(window or 0), float(lam), float(eps), float(out_scale), int(n_splits),
+        _dev(seg_len, "seg_len", torch.int32) if below > 0 else 0, int(below), _stream()), "diff_attention")
+    return out
+
+
+def diff_attention_tiles_takes(dtype: torch.dtype, page_size: int, dim: int, vdim: int) -> bool:
+    """Whether the matrix-core kernel for portions takes these sizes."""
+    return dtype == torch.bfloat16 and bool(library().imparo_diff_attention_tiles_takes(int(page_size), int(dim), int(vdim)))
+
+
+def diff_attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gate: Optional[torch.Tensor],
+                         gate_ld: int, out: torch.Tensor, positions: torch.Tensor, seg_start: torch.Tensor,
+                         seg_len: torch.Tensor, max_seg_len: int, block_table: torch.Tensor, scale: float,
+                         window: Optional[int], lam: float, eps: float, out_scale: float, min_len: int = 1) -> torch.Tensor:
+    """Differential attention on the matrix cores for the rows that bring at least `min_len` tokens (bfloat16;
+    sizes as diff_attention_tiles_takes says); the other rows' outputs are left as they are."""
+    n, heads, two, dim = q.shape
+    n_pages, kv2, page_size, kdim = k_cache.shape
+    kv_heads, vdim = v_cache.shape[1], v_cache.shape[3]
+    n_rows = seg_start.shape[0]
+    if two != 2 or kdim != dim or kv2 != 2 * kv_heads or heads % kv_heads:
+        raise KernelArgumentError("diff_attention_tiles: queries [tokens, heads, 2, dim], keys [pages, 2 kv_heads, page, dim]")
+    if not diff_attention_tiles_takes(q.dtype, page_size, dim, vdim):
+        raise KernelArgumentError(f"diff_attention_tiles: bfloat16, pages of a multiple of 16, dim and vdim multiples of 4 "
+                                  f"up to 128; got {q.dtype}, pages of {page_size}, {dim} and {vdim}")
+    if gate is not None and (gate.dtype != torch.float32 or gate.device != q.device):
+        raise KernelArgumentError("diff_attention_tiles: the gate's logits are float32 on the GPU")
+    _check(library().imparo_diff_attention_tiles(
+        _dev(q, "q", torch.bfloat16), _dev(k_cache, "k cache", torch.bfloat16),
+        _dev(v_cache, "v cache", torch.bfloat16, (n_pages, kv_heads, page_size, vdim)), 0 if gate is None else gate.data_ptr(),
+        int(gate_ld), _dev(out, "attention out", torch.bfloat16, (n, heads * vdim)), _dev(positions, "positions", torch.int32, (n,)),
+        _dev(seg_start, "seg_start", torch.int32, (n_rows,)), _dev(seg_len, "seg_len", torch.int32, (n_rows,)),
+        _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size, n_rows, int(max_seg_len), heads,
+        kv_heads, dim, vdim, n_pages, float(scale), int(window or 0), float(lam), float(eps), float(out_scale),
+        int(min_len), _stream()), "diff_attention_tiles")
     return out

@@ -122,13 +122,25 @@ class DifferentialAttention:
                            k_cache if owns_cache else None, v_cache if owns_cache else None, self.heads,
                            self.kv_heads, self.dim, self.vdim, self.temp_coef, self.temp_every)
         o = ctx.workspace.get("attn_out", (T, self.heads * self.vdim), ctx.dtype, alias="mixer_mid")
-        n_splits = self._splits(ctx, T)
-        part = None
-        if n_splits > 1:
-            part = ctx.workspace.get("diff_attn_part", (T * self.heads * n_splits * (2 * self.vdim + 4),), torch.float32)
         gate = rows[:, self.gate_at:] if self.gated else None
-        ops.diff_attention(q, k_cache, v_cache, gate, rows.shape[1], o, ctx.positions, ctx.row_of_token, table,
-                           self.scale, self.window, self.lam, self.eps, 1.0 - self.diff, part, n_splits)
+        # rows that bring portions go to the matrix cores where the sizes allow; single tokens to the wave
+        # kernel, their keys in splits when few of them walk long contexts
+        tiles = (ctx.max_seg_len > 1 and ctx.single_rows is not None
+                 and ops.diff_attention_tiles_takes(ctx.dtype, ctx.page_size, self.dim, self.vdim))
+        if tiles:
+            ops.diff_attention_tiles(q, k_cache, v_cache, gate, rows.shape[1], o, ctx.positions, ctx.seg_start,
+                                     ctx.seg_len, ctx.max_seg_len, table, self.scale, self.window, self.lam, self.eps,
+                                     1.0 - self.diff, min_len=2)
+        if not tiles or ctx.n_single_rows:
+            singles = ctx.n_single_rows if tiles else T
+            n_splits = self._splits(ctx, singles)
+            part = None
+            if n_splits > 1:
+                part = ctx.workspace.get("diff_attn_part", (T * self.heads * n_splits * (2 * self.vdim + 4),),
+                                         torch.float32)
+            ops.diff_attention(q, k_cache, v_cache, gate, rows.shape[1], o, ctx.positions, ctx.row_of_token, table,
+                               self.scale, self.window, self.lam, self.eps, 1.0 - self.diff, part, n_splits,
+                               seg_len=ctx.seg_len if tiles else None, below=2 if tiles else 0)
         if o.dtype != self.out.in_dtype:
             raise ValueError("the output projection's weight dtype differs from the attention output's")
         return self.out(ctx, o, torch.float32, "mixer_out", sliced_ok=True, into=ctx.stream)

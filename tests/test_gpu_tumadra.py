@@ -284,6 +284,58 @@ def test_differential_attention_finds_a_far_key(dtype):
         assert float((out - ref).abs().max()) < tol, f"{n_splits} splits"
 
 
+@pytest.mark.parametrize("H,G,D,V,page", [(4, 2, 16, 32, 16), (3, 1, 24, 40, 64), (1, 1, 8, 8, 16), (4, 1, 64, 128, 32),
+                                          (2, 2, 36, 20, 16)])
+def test_differential_attention_matrix_core_kernel(H, G, D, V, page):
+    """The kernel for portions (bfloat16): a portion of 403 queries behind 297 cached keys, beside a row of
+    one token that it must leave alone and a short row of three; a far key that the second map singles out."""
+    from imparo_amd.kernels import ops
+    g = torch.Generator().manual_seed(H * 10 + D)
+    n_ctx, cut = 700, 297
+    q = torch.randn(n_ctx, H, 2, D, generator=g)
+    k = torch.randn(n_ctx, G, 2, D, generator=g)
+    v = torch.randn(n_ctx, G, V, generator=g)
+    gate = torch.randn(n_ctx, H * V, generator=g)
+    k[5, :, 1] = 4.0 * q[-1, 0, 1] / q[-1, 0, 1].norm()
+    q[-3:, :, 1] = 3.0 * q[-1, 0, 1]
+    v[5] = 5.0
+    q, k, v = [t.to(torch.bfloat16).float() for t in (q, k, v)]
+    scale, lam, diff, eps = 1.0 / math.sqrt(D), 0.65, 0.35, 1e-5
+    ref = plain.differential_core(q, k, v, torch.arange(n_ctx), scale, lam, diff, eps) * torch.sigmoid(gate)
+    n_pages = 2 * (-(-n_ctx // page)) + 2
+    order = list(range(n_pages))
+    random.Random(D).shuffle(order)
+    per = -(-n_ctx // page)
+    # request 0 holds all 700 keys; request 1 holds the first 3 of the same sequence in pages of its own
+    table = i32([order[:per], order[per:2 * per]])
+    k_cache = torch.zeros(n_pages, 2 * G, page, D, device=DEV, dtype=torch.bfloat16)
+    v_cache = torch.zeros(n_pages, G, page, V, device=DEV, dtype=torch.bfloat16)
+    rows = torch.cat([q.reshape(n_ctx, -1), k.reshape(n_ctx, -1), v.reshape(n_ctx, -1), gate], dim=1)
+    store = lambda sel, row: ops.diff_qkv_store(
+        dev(rows[sel]), i32(sel), i32([row] * len(sel)), table, page,
+        torch.empty(len(sel), H, 2, D, device=DEV, dtype=torch.bfloat16), k_cache, v_cache, H, G, D, V, 0.0, 0)
+    store(list(range(cut)), 0)
+    # the step: request 0's last 403 tokens, a single token of request 0's twin... kept simple: request 1 brings 3 tokens
+    sel = list(range(cut, n_ctx)) + [0, 1, 2]
+    row_of = [0] * (n_ctx - cut) + [1] * 3
+    q_dev = torch.empty(len(sel), H, 2, D, device=DEV, dtype=torch.bfloat16)
+    ops.diff_qkv_store(dev(rows[sel]), i32(sel), i32(row_of), table, page, q_dev, k_cache, v_cache, H, G, D, V, 0.0, 0)
+    out = torch.full((len(sel), H * V), 9.0, device=DEV, dtype=torch.bfloat16)
+    ops.diff_attention_tiles(q_dev, k_cache, v_cache, dev(gate[sel]), H * V, out, i32(sel), i32([0, n_ctx - cut]),
+                             i32([n_ctx - cut, 3]), n_ctx - cut, table, scale, None, lam, eps, 1.0 - diff, min_len=2)
+    got = out.float().cpu()
+    assert float((got - ref[sel]).abs().max()) < 4e-2
+    # with min_len 4 the short row is left alone
+    out.fill_(9.0)
+    ops.diff_attention_tiles(q_dev, k_cache, v_cache, dev(gate[sel]), H * V, out, i32(sel), i32([0, n_ctx - cut]),
+                             i32([n_ctx - cut, 3]), n_ctx - cut, table, scale, None, lam, eps, 1.0 - diff, min_len=4)
+    assert float((out[:-3].float().cpu() - ref[sel[:-3]]).abs().max()) < 4e-2 and bool((out[-3:] == 9.0).all())
+    # and the wave kernel takes exactly the rows below a length
+    ops.diff_attention(q_dev, k_cache, v_cache, dev(gate[sel]), H * V, out, i32(sel), i32(row_of), table, scale, None, lam,
+                       eps, 1.0 - diff, None, 1, seg_len=i32([n_ctx - cut, 3]), below=4)
+    assert float((out.float().cpu() - ref[sel]).abs().max()) < 4e-2
+
+
 # ------------------------------------------------------------------ the model in the engine
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
