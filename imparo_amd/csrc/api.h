@@ -246,14 +246,14 @@ int imparo_causal_conv(const float* u, int u_ld, const float* weight, const floa
                        const int32_t* slot, void* out, int out_dtype, int n_tokens, int n_rows, int channels, int taps,
                        int silu, int single_tokens, imparo_stream stream);
 // S[c, n] <- exp(dt A[c, n]) S[c, n] + dt x[c] B[n]; y[c] = sum_n S[c, n] C[n] + D[c] x[c]; out = y * silu(z);
-// dt = softplus(dt_raw). bc rows are [B | C] float32; state [slots, channels, n_state] float32. n_chunks 1:
+// dt = softplus(dt_raw), taken in place (dt_raw [n_tokens, channels] holds the steps afterwards). bc rows are [B | C] float32; state [slots, channels, n_state] float32. n_chunks 1:
 // every segment in one piece; more (at least ceil(longest segment / imparo_selective_scan_chunk())): chunks of a
 // segment run side by side through scratch, n_rows * (n_chunks * channels * (n_state + 1) + channels * n_state) floats.
 int imparo_selective_scan_chunk(void);
-int imparo_selective_scan(const float* dt_raw, const void* x, const float* bc, const float* z, int z_ld,
+int imparo_selective_scan(float* dt_raw, const void* x, const float* bc, const float* z, int z_ld,
                           const float* A, const float* D, float* state, const int32_t* seg_start,
                           const int32_t* seg_len, const int32_t* slot, void* out, int dtype, float* scratch,
-                          int n_chunks, int n_rows, int channels, int n_state, imparo_stream stream);
+                          int n_chunks, int n_tokens, int n_rows, int channels, int n_state, imparo_stream stream);
 
 // ---- differential attention (two softmax maps a head over shared values)
 // rows_in float32 [tokens, ld] = [q: heads x 2 x dim | k: kv_heads x 2 x dim | v: kv_heads x vdim | ...];

@@ -326,6 +326,39 @@ __device__ __forceinline__ da_s16x4 da_pack4(float a, float b, float c, float d)
     return r;
 }
 
+// The operands of one tile of 32 keys: for each of its two blocks of 16 keys whether its page is there, and
+// the K rows (both maps) as the first product's left operand.
+template <int D16>
+struct DaKeys {
+    da_s16x4 k[2][2][D16];       // [map][block of 16 keys][16 dims]
+    long long vbase[2];
+    bool there[2];
+};
+
+template <int D16>
+__device__ __forceinline__ void da_load_keys(DaKeys<D16>& t, const bf16_t* __restrict__ k_cache,
+                                             const int32_t* __restrict__ table, int k0, int pos_last, int page_size,
+                                             int n_pages, int kv_heads, int g, int dim, int vdim, int col, int quad) {
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+        const int key0 = k0 + mb * 16;                       // a block of 16 keys lies in one page
+        const int page = key0 <= pos_last ? table[key0 / page_size] : -1;
+        t.there[mb] = page >= 0 && page < n_pages;
+        const long long pg = t.there[mb] ? page : 0;          // a block that is not there reads page 0 and counts for nothing
+        const long long kbase = ((pg * 2 * kv_heads + 2 * g) * page_size + (key0 % page_size)) * dim;
+        t.vbase[mb] = ((pg * kv_heads + g) * page_size + (key0 % page_size)) * (long long)vdim;
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+            for (int kk = 0; kk < D16; ++kk) {
+                const int d = min(kk * 16 + quad * 4, dim - 4);          // dims past the head repeat its end; the query holds zeros there
+                t.k[m][mb][kk] = *reinterpret_cast<const da_s16x4*>(k_cache + kbase + ((long long)m * page_size + col) * dim + d);
+            }
+    }
+}
+
+// D16, V16: blocks of 16 of dim and of vdim that the registers hold (4 or 8).
+template <int D16, int V16>
 __global__ __launch_bounds__(256) void k_diff_attention_tiles(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const float* __restrict__ gate, int gate_ld, bf16_t* __restrict__ out, const int32_t* __restrict__ positions,
@@ -348,41 +381,47 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
     const int lo_first = window > 0 ? max(0, pos_first + 1 - window) : 0;
     const int g = h / (heads / kv_heads);
-    const int dim16 = (dim + 15) >> 4, vd16 = (vdim + 15) >> 4;
+    const int vd16 = (vdim + 15) >> 4;
     const int32_t* table = block_table + (size_t)r * table_stride;
 
-    // Q^T operands: query `col`, dims 16 kk + 4 quad .. + 3, both maps
-    da_s16x4 qf[2][DAM_MAX16];
+    // Q^T operands: query `col`, dims 16 kk + 4 quad .. + 3, both maps; zeros past the head's dims
+    da_s16x4 qf[2][D16];
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
-        for (int kk = 0; kk < DAM_MAX16; ++kk) {
+        for (int kk = 0; kk < D16; ++kk) {
             const int d = kk * 16 + quad * 4;
-            const bool on = kk < dim16 && d < dim;
-            const bf16_t* src = q + (((size_t)t * heads + h) * 2 + m) * dim + (on ? d : 0);
-            const da_s16x4 v = *reinterpret_cast<const da_s16x4*>(src);
-            qf[m][kk] = on ? v : da_s16x4{0, 0, 0, 0};
+            const da_s16x4 v = *reinterpret_cast<const da_s16x4*>(q + (((size_t)t * heads + h) * 2 + m) * dim + min(d, dim - 4));
+            qf[m][kk] = d < dim ? v : da_s16x4{0, 0, 0, 0};
         }
-    da_f32x4 o[2][DAM_MAX16];
+    da_f32x4 o[2][V16];
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
-        for (int vb = 0; vb < DAM_MAX16; ++vb) o[m][vb] = da_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int vb = 0; vb < V16; ++vb) o[m][vb] = da_f32x4{0.f, 0.f, 0.f, 0.f};
     float mx[2] = {-INFINITY, -INFINITY}, sum[2] = {0.f, 0.f};
 
-    for (int k0 = (lo_first / 32) * 32; k0 <= pos_last; k0 += 32) {
-        // the two blocks of 16 keys of this tile lie in one page each
-        long long kbase[2], vbase[2];
-        bool there[2];
+    DaKeys<D16> cur, nxt;
+    int k0 = (lo_first / 32) * 32;
+    da_load_keys<D16>(cur, k_cache, table, k0, pos_last, page_size, n_pages, kv_heads, g, dim, vdim, col, quad);
+    for (; k0 <= pos_last; k0 += 32) {
+        // this tile's values and the next tile's keys are asked for before this tile's products begin
+        da_s16x4 vt[2][V16];
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-            const int key0 = k0 + mb * 16;
-            const int page = key0 <= pos_last ? table[key0 / page_size] : -1;
-            there[mb] = page >= 0 && page < n_pages;
-            const long long pg = there[mb] ? page : 0;
-            kbase[mb] = ((pg * 2 * kv_heads + 2 * g) * page_size + (key0 % page_size)) * dim;
-            vbase[mb] = ((pg * kv_heads + g) * page_size + (key0 % page_size)) * (long long)vdim;
-        }
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int vb = 0; vb < V16; ++vb) {
+                if (vb >= vd16) continue;
+                // keys 4 quad .. + 3 of the block, value dimension 16 vb + col: four rows of V, one value each
+                const int d = min(vb * 16 + col, vdim - 1);
+                const bf16_t* src = v_cache + cur.vbase[mb] + (long long)(quad * 4) * vdim + d;
+                vt[mb][vb][0] = (short)src[0];
+                vt[mb][vb][1] = (short)src[vdim];
+                vt[mb][vb][2] = (short)src[2 * vdim];
+                vt[mb][vb][3] = (short)src[3 * vdim];
+            }
+        da_load_keys<D16>(nxt, k_cache, table, k0 + 32, pos_last, page_size, n_pages, kv_heads, g, dim, vdim, col, quad);
+
         da_s16x4 pb[2][2];                                   // P^T operands: [map][block of 16 keys]
         float corr[2];
 #pragma unroll
@@ -391,16 +430,8 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-                for (int kk = 0; kk < DAM_MAX16; ++kk) {
-                    if (kk < dim16) {
-                        const int d = kk * 16 + quad * 4;
-                        const bool on = d < dim;
-                        // key row `col` of the block, map m, dims d .. d + 3
-                        const bf16_t* src = k_cache + kbase[mb] + ((long long)m * page_size + col) * dim + (on ? d : 0);
-                        const da_s16x4 kv = *reinterpret_cast<const da_s16x4*>(src);
-                        sc[mb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(on ? kv : da_s16x4{0, 0, 0, 0}, qf[m][kk], sc[mb], 0, 0, 0);
-                    }
-                }
+                for (int kk = 0; kk < D16; ++kk)
+                    sc[mb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(cur.k[m][mb][kk], qf[m][kk], sc[mb], 0, 0, 0);
             // a lane holds keys k0 + 16 mb + 4 quad + i of query `col`
             float tile_max = -INFINITY;
 #pragma unroll
@@ -408,7 +439,7 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int key = k0 + mb * 16 + quad * 4 + i;
-                    const bool seen = there[mb] && key <= pos && key >= lo;
+                    const bool seen = cur.there[mb] && key <= pos && key >= lo;
                     sc[mb][i] = seen ? sc[mb][i] * scale : -INFINITY;
                     tile_max = fmaxf(tile_max, sc[mb][i]);
                 }
@@ -434,7 +465,7 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
             for (int mb = 0; mb < 2; ++mb) pb[m][mb] = da_pack4(p[mb][0], p[mb][1], p[mb][2], p[mb][3]);
         }
 #pragma unroll
-        for (int vb = 0; vb < DAM_MAX16; ++vb) {
+        for (int vb = 0; vb < V16; ++vb) {
             if (vb < vd16) {
 #pragma unroll
                 for (int m = 0; m < 2; ++m) {
@@ -443,33 +474,27 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
                     o[m][vb][2] *= corr[m];
                     o[m][vb][3] *= corr[m];
                 }
-                const int d = vb * 16 + col;                   // V^T row of this lane
-                const bool on_d = d < vdim;
+                const bool on_d = vb * 16 + col < vdim;
 #pragma unroll
                 for (int mb = 0; mb < 2; ++mb) {
-                    // keys 4 quad .. + 3 of the block, value dimension d: four rows of V, one value each
-                    const bf16_t* src = v_cache + vbase[mb] + (long long)(quad * 4) * vdim + (on_d ? d : 0);
-                    da_s16x4 vt;
-                    vt[0] = (short)src[0];
-                    vt[1] = (short)src[vdim];
-                    vt[2] = (short)src[2 * vdim];
-                    vt[3] = (short)src[3 * vdim];
+                    da_s16x4 v = vt[mb][vb];
                     const int key = k0 + mb * 16 + quad * 4;         // what lies past the last query's position is not a value yet
-                    if (key + 1 > pos_last) vt[1] = 0;
-                    if (key + 2 > pos_last) vt[2] = 0;
-                    if (key + 3 > pos_last) vt[3] = 0;
-                    if (!(on_d && there[mb]) || key > pos_last) vt = da_s16x4{0, 0, 0, 0};
-                    o[0][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt, pb[0][mb], o[0][vb], 0, 0, 0);
-                    o[1][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt, pb[1][mb], o[1][vb], 0, 0, 0);
+                    if (key + 1 > pos_last) v[1] = 0;
+                    if (key + 2 > pos_last) v[2] = 0;
+                    if (key + 3 > pos_last) v[3] = 0;
+                    if (!(on_d && cur.there[mb]) || key > pos_last) v = da_s16x4{0, 0, 0, 0};
+                    o[0][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v, pb[0][mb], o[0][vb], 0, 0, 0);
+                    o[1][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v, pb[1][mb], o[1][vb], 0, 0, 0);
                 }
             }
         }
+        cur = nxt;
     }
     // finish: a lane holds value dimensions 16 vb + 4 quad + i of query `col`
     const float i1 = sum[0] > 0.f ? 1.0f / sum[0] : 0.f, i2 = sum[1] > 0.f ? 1.0f / sum[1] : 0.f;
     float ss = 0.f;
 #pragma unroll
-    for (int vb = 0; vb < DAM_MAX16; ++vb)
+    for (int vb = 0; vb < V16; ++vb)
         if (vb < vd16) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -486,7 +511,7 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
         const float* gt = gate ? gate + (size_t)t * gate_ld + (size_t)h * vdim : nullptr;
         bf16_t* dst = out + ((size_t)t * heads + h) * vdim;
 #pragma unroll
-        for (int vb = 0; vb < DAM_MAX16; ++vb)
+        for (int vb = 0; vb < V16; ++vb)
             if (vb < vd16) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -524,10 +549,16 @@ extern "C" int imparo_diff_attention_tiles(const void* q, const void* k_cache, c
     const int tiles = (max_seg_len + DAM_TILE - 1) / DAM_TILE;
     if (tiles > 65535) return IMPARO_BAD_ARGUMENT;
     dim3 grid(n_rows, tiles, heads);
-    k_diff_attention_tiles<<<grid, 256, 0, (hipStream_t)stream>>>(
-        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, gate, gate_ld, (bf16_t*)out, positions, seg_start,
-        seg_len, block_table, table_stride, page_size, heads, kv_heads, dim, vdim, n_pages, scale, window, lambda, eps,
-        out_scale, min_len);
+#define DAM_LAUNCH(D16, V16)                                                                                             \
+    k_diff_attention_tiles<D16, V16><<<grid, 256, 0, (hipStream_t)stream>>>(                                              \
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, gate, gate_ld, (bf16_t*)out, positions, seg_start, \
+        seg_len, block_table, table_stride, page_size, heads, kv_heads, dim, vdim, n_pages, scale, window, lambda, eps,   \
+        out_scale, min_len)
+    if (dim <= 64 && vdim <= 64) DAM_LAUNCH(4, 4);
+    else if (dim <= 64) DAM_LAUNCH(4, 8);
+    else if (vdim <= 64) DAM_LAUNCH(8, 4);
+    else DAM_LAUNCH(8, 8);
+#undef DAM_LAUNCH
     return launch_status();
 }
 

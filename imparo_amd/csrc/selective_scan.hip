@@ -139,8 +139,21 @@ extern "C" int imparo_causal_conv(const float* u, int u_ld, const float* weight,
 
 extern "C" int imparo_selective_scan_chunk(void) { return SCAN_CHUNK; }
 
+// dt <- softplus(dt) in place, once per (token, channel): the scan's lanes that share a channel would each
+// take it again, in both of its launches.
+__global__ void k_softplus_rows(float* __restrict__ dt, long long n) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dt[i] = softplus_f32(dt[i]);
+}
+
+// exp of a decay's exponent: the library's in float32, the hardware's exp2 where the engine rounds its
+// activations to bfloat16 anyway
+template <typename TX> __device__ __forceinline__ float decay_exp(float v);
+template <> __device__ __forceinline__ float decay_exp<float>(float v) { return expf(v); }
+template <> __device__ __forceinline__ float decay_exp<bf16_t>(float v) { return __expf(v); }
+
 template <typename TX, typename TOut, int SPL, int UNR, bool EMIT>
-__device__ __forceinline__ float scan_walk(const float* __restrict__ dt_raw, const TX* __restrict__ x,
+__device__ __forceinline__ float scan_walk(const float* __restrict__ dt_raw /* steps, softplus taken */, const TX* __restrict__ x,
                                            const float* __restrict__ bc, const float* __restrict__ z, int z_ld,
                                            TOut* __restrict__ out, float (&S)[SPL], const float (&a)[SPL], float d_skip,
                                            size_t t_first, int count, int channels, int cc, int n_state, int lp, int ln,
@@ -164,14 +177,14 @@ __device__ __forceinline__ float scan_walk(const float* __restrict__ dt_raw, con
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
             const bool on = i + u < count;
-            const float step = on ? softplus_f32(dt[u]) : 0.f;
+            const float step = on ? dt[u] : 0.f;
             const float dx = step * xv[u];
             dt_sum += step;
             float y = 0.f;
 #pragma unroll
             for (int j = 0; j < SPL; ++j) {
                 const bool has = ln + j * lp < n_state;
-                const float s_new = expf(step * a[j]) * S[j] + dx * b[u][j];
+                const float s_new = decay_exp<TX>(step * a[j]) * S[j] + dx * b[u][j];
                 S[j] = has ? s_new : 0.f;
                 y += has ? s_new * cv[u][j] : 0.f;
             }
@@ -263,7 +276,7 @@ __global__ void k_selective_scan(const float* __restrict__ dt_raw, const TX* __r
 #pragma unroll
         for (int j = 0; j < SPL; ++j) {
             const int n = min(ln + j * lp, n_state - 1);
-            S[j] = ln + j * lp < n_state ? expf(sum * a[j]) * S[j] + ends[n] : 0.f;
+            S[j] = ln + j * lp < n_state ? decay_exp<TX>(sum * a[j]) * S[j] + ends[n] : 0.f;
         }
     }
     const int first = chunks > 1 ? k * SCAN_CHUNK : 0;
@@ -280,10 +293,10 @@ __global__ void k_selective_scan(const float* __restrict__ dt_raw, const TX* __r
 }
 
 template <typename TX, typename TOut>
-static int launch_scan(const float* dt_raw, const void* x, const float* bc, const float* z, int z_ld, const float* A,
+static int launch_scan(float* dt_raw, const void* x, const float* bc, const float* z, int z_ld, const float* A,
                        const float* D, float* state, const int32_t* seg_start, const int32_t* seg_len,
-                       const int32_t* slot, void* out, float* scratch, int n_chunks, int n_rows, int channels,
-                       int n_state, hipStream_t s) {
+                       const int32_t* slot, void* out, float* scratch, int n_chunks, int n_tokens, int n_rows,
+                       int channels, int n_state, hipStream_t s) {
     int lp = 1;
     while (lp < n_state && lp < WAVE) lp <<= 1;
     const int spl = (n_state + lp - 1) / lp;
@@ -291,6 +304,9 @@ static int launch_scan(const float* dt_raw, const void* x, const float* bc, cons
     const int per_block = threads / lp;
     dim3 grid(n_rows, (channels + per_block - 1) / per_block, n_chunks);
     if (grid.y > 65535 || grid.z > 65535) return IMPARO_BAD_ARGUMENT;
+    const long long n_dt = (long long)n_tokens * channels;
+    k_softplus_rows<<<(unsigned)((n_dt + 255) / 256), 256, 0, s>>>(dt_raw, n_dt);
+    if (launch_status()) return IMPARO_LAUNCH_FAILED;
 #define SCAN_LAUNCH(N, U)                                                                                             \
     do {                                                                                                              \
         if (n_chunks > 1) {                                                                                           \
@@ -312,28 +328,30 @@ static int launch_scan(const float* dt_raw, const void* x, const float* bc, cons
     return launch_status();
 }
 
-// dt_raw [tokens, channels] float32 (the step projection with its bias, before softplus); x [tokens,
+// dt_raw [tokens, channels] float32 (the step projection with its bias, before softplus; softplus is taken in
+// place, so the array holds the steps afterwards); x [tokens,
 // channels] in `dtype`; bc [tokens, 2 n_state] float32 (B then C); z rows z_ld floats apart; A, D float32
 // (A = -exp(A_log), [channels, n_state]); state [slots, channels, n_state] float32; out [tokens, channels]
 // in `dtype`. n_state at most 512. n_chunks 1: every segment is walked in one piece. More (at least
 // ceil(longest segment / imparo_selective_scan_chunk())): segments are walked in chunks side by side through
 // `scratch`, n_rows * (n_chunks * channels * (n_state + 1) + channels * n_state) floats.
-extern "C" int imparo_selective_scan(const float* dt_raw, const void* x, const float* bc, const float* z, int z_ld,
+extern "C" int imparo_selective_scan(float* dt_raw, const void* x, const float* bc, const float* z, int z_ld,
                                      const float* A, const float* D, float* state, const int32_t* seg_start,
                                      const int32_t* seg_len, const int32_t* slot, void* out, int dtype, float* scratch,
-                                     int n_chunks, int n_rows, int channels, int n_state, imparo_stream stream) {
+                                     int n_chunks, int n_tokens, int n_rows, int channels, int n_state,
+                                     imparo_stream stream) {
     if (!dt_raw || !x || !bc || !z || !A || !D || !state || !seg_start || !seg_len || !slot || !out)
         return IMPARO_BAD_ARGUMENT;
-    if (n_rows < 0 || channels <= 0 || n_state <= 0 || n_state > 512 || z_ld < channels) return IMPARO_BAD_ARGUMENT;
+    if (n_rows < 0 || n_tokens < 0 || channels <= 0 || n_state <= 0 || n_state > 512 || z_ld < channels) return IMPARO_BAD_ARGUMENT;
     if (n_chunks < 1 || (n_chunks > 1 && !scratch)) return IMPARO_BAD_ARGUMENT;
-    if (n_rows == 0) return IMPARO_OK;
+    if (n_rows == 0 || n_tokens == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == IMPARO_F32)
         return launch_scan<float, float>(dt_raw, x, bc, z, z_ld, A, D, state, seg_start, seg_len, slot, out, scratch,
-                                         n_chunks, n_rows, channels, n_state, s);
+                                         n_chunks, n_tokens, n_rows, channels, n_state, s);
     if (dtype == IMPARO_BF16)
         return launch_scan<bf16_t, bf16_t>(dt_raw, x, bc, z, z_ld, A, D, state, seg_start, seg_len, slot, out, scratch,
-                                           n_chunks, n_rows, channels, n_state, s);
+                                           n_chunks, n_tokens, n_rows, channels, n_state, s);
     return IMPARO_BAD_ARGUMENT;
 }
 

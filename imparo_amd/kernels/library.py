@@ -55,7 +55,7 @@ _SIGNATURES = {
     "imparo_token_shift": [P, P, P, P, P, P, P, P, I, I, I, I, P],
     "imparo_poly_norm": [P, I, P, P, I, I, I, I, F, P],
     "imparo_causal_conv": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
-    "imparo_selective_scan": [P, P, P, P, I, P, P, P, P, P, P, P, I, P, I, I, I, I, P],
+    "imparo_selective_scan": [P, P, P, P, I, P, P, P, P, P, P, P, I, P, I, I, I, I, I, P],
     "imparo_selective_scan_chunk": [],
     "imparo_diff_qkv_store": [P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
     "imparo_diff_attention_split": [],

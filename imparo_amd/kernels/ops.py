@@ -627,7 +627,8 @@ def selective_scan(dt_raw: torch.Tensor, x: torch.Tensor, bc: torch.Tensor, z: t
                    slot: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tensor] = None,
                    n_chunks: int = 1) -> torch.Tensor:
     """The selective scan of every request's segment, continued from its state [slots, channels, n_state]
-    (float32), which is advanced. dt_raw [tokens, channels] float32 before softplus; x and out [tokens,
+    (float32), which is advanced. dt_raw [tokens, channels] float32 before softplus (taken in place: the
+    array holds the steps afterwards); x and out [tokens,
     channels] in one dtype; bc [tokens, 2 n_state] float32; z a float32 view whose rows lie z_ld apart.
     `n_chunks` > 1 (at least ceil(longest segment / selective_scan_chunk())): the chunks of a segment run
     side by side through `scratch` (selective_scan_scratch floats); the caller knows the longest segment."""
@@ -645,7 +646,7 @@ def selective_scan(dt_raw: torch.Tensor, x: torch.Tensor, bc: torch.Tensor, z: t
         _dev(seg_start, "seg_start", torch.int32, (n_rows,)), _dev(seg_len, "seg_len", torch.int32, (n_rows,)),
         _dev(slot, "slot", torch.int32, (n_rows,)), _dev(out, "scan out", x.dtype, (n, channels)), _code(x, "scan x"),
         _dev(scratch, "scan scratch", torch.float32) if n_chunks > 1 else 0, int(n_chunks),
-        n_rows, channels, n_state, _stream()), "selective_scan")
+        n, n_rows, channels, n_state, _stream()), "selective_scan")
     return out
 
 
