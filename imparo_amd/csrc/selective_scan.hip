@@ -128,7 +128,8 @@ extern "C" int imparo_causal_conv(const float* u, int u_ld, const float* weight,
 // channel's states, SPL states a lane (n = lane + j * LP). Tokens are walked in order, UNR at a time:
 // their inputs are asked for together, from clamped addresses, and a token past the end walks with a
 // step of zero, which leaves the state as it is. A token's sum_n S[n] C[n] is added up across the LP
-// lanes by a butterfly, the same order whatever the batch.
+// lanes by a butterfly, the same order whatever the batch; lane u of the channel then gates and stores
+// the batch's token u (UNR never passes LP).
 //
 // A long segment is cut into chunks of SCAN_CHUNK tokens that run side by side: k_scan_chunk_state walks
 // every chunk but the last from a zero state and leaves its end state E_k and the sum of its steps (the
@@ -160,13 +161,15 @@ __device__ __forceinline__ float scan_walk(const float* __restrict__ dt_raw /* s
                                            bool live) {
     float dt_sum = 0.f;
     for (int i = 0; i < count; i += UNR) {
-        float dt[UNR], xv[UNR], zv[UNR], b[UNR][SPL], cv[UNR][SPL];
+        float dt[UNR], xv[UNR], b[UNR][SPL], cv[UNR][SPL];
+        // lane u of a channel's lanes finishes token i + u of the batch: its gate is all it has to ask for
+        const bool finisher = EMIT && ln < UNR && live && i + ln < count;
+        const float z_mine = EMIT ? z[(t_first + (size_t)min(i + min(ln, UNR - 1), count - 1)) * z_ld + cc] : 0.f;
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
             const size_t t = t_first + (size_t)min(i + u, count - 1);
             dt[u] = dt_raw[t * channels + cc];
             xv[u] = load_f32<TX>(x, t * channels + cc);
-            zv[u] = EMIT ? z[t * z_ld + cc] : 0.f;
 #pragma unroll
             for (int j = 0; j < SPL; ++j) {
                 const int nn = min(ln + j * lp, n_state - 1);
@@ -174,6 +177,7 @@ __device__ __forceinline__ float scan_walk(const float* __restrict__ dt_raw /* s
                 cv[u][j] = EMIT ? bc[t * 2 * n_state + n_state + nn] : 0.f;
             }
         }
+        float y_mine = 0.f, x_mine = 0.f;
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
             const bool on = i + u < count;
@@ -189,12 +193,14 @@ __device__ __forceinline__ float scan_walk(const float* __restrict__ dt_raw /* s
                 y += has ? s_new * cv[u][j] : 0.f;
             }
             if (EMIT) {
-                for (int off = lp >> 1; off > 0; off >>= 1) y += __shfl_xor(y, off, WAVE);
-                if (ln == 0 && live && on) {
-                    y += d_skip * xv[u];
-                    store_f32<TOut>(out, (t_first + i + u) * channels + cc, y * silu_f32(zv[u]));
-                }
+                for (int off = lp >> 1; off > 0; off >>= 1) y += __shfl_xor(y, off, WAVE);   // every lane of the channel has the sum
+                y_mine = ln == u ? y : y_mine;
+                x_mine = ln == u ? xv[u] : x_mine;
             }
+        }
+        if (finisher) {
+            const float gate = z_mine / (1.0f + decay_exp<TX>(-z_mine));
+            store_f32<TOut>(out, (t_first + i + ln) * channels + cc, (y_mine + d_skip * x_mine) * gate);
         }
     }
     return dt_sum;
@@ -319,7 +325,10 @@ static int launch_scan(float* dt_raw, const void* x, const float* bc, const floa
                                                                   seg_start, seg_len, slot, (TOut*)out, scratch,      \
                                                                   n_rows, n_chunks, channels, n_state, lp);           \
     } while (0)
-    if (spl == 1) SCAN_LAUNCH(1, 8);
+    if (spl == 1 && lp >= 8) SCAN_LAUNCH(1, 8);        // a batch of tokens is finished by as many lanes of the channel
+    else if (spl == 1 && lp == 4) SCAN_LAUNCH(1, 4);
+    else if (spl == 1 && lp == 2) SCAN_LAUNCH(1, 2);
+    else if (spl == 1) SCAN_LAUNCH(1, 1);
     else if (spl == 2) SCAN_LAUNCH(2, 4);
     else if (spl <= 4) SCAN_LAUNCH(4, 2);
     else if (spl <= 8) SCAN_LAUNCH(8, 1);
