@@ -18,7 +18,7 @@
 #define DA_WAVES 4
 #define DA_MAX_DIM 256
 #define DA_MAX_VDIM 512
-#define DA_SPLIT 256
+#define DA_SPLIT 128
 
 extern "C" int imparo_diff_attention_split(void) { return DA_SPLIT; }
 

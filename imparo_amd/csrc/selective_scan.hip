@@ -154,11 +154,11 @@ template <> __device__ __forceinline__ float decay_exp<float>(float v) { return 
 template <> __device__ __forceinline__ float decay_exp<bf16_t>(float v) { return __expf(v); }
 
 template <typename TX, typename TOut, int SPL, int UNR, bool EMIT>
-__device__ __forceinline__ float scan_walk(const float* __restrict__ dt_raw /* steps, softplus taken */, const TX* __restrict__ x,
+__device__ __forceinline__ float scan_walk(const float* __restrict__ dt_raw /* steps; raw == true: before softplus */, const TX* __restrict__ x,
                                            const float* __restrict__ bc, const float* __restrict__ z, int z_ld,
                                            TOut* __restrict__ out, float (&S)[SPL], const float (&a)[SPL], float d_skip,
                                            size_t t_first, int count, int channels, int cc, int n_state, int lp, int ln,
-                                           bool live) {
+                                           bool live, bool raw = false) {
     float dt_sum = 0.f;
     for (int i = 0; i < count; i += UNR) {
         float dt[UNR], xv[UNR], b[UNR][SPL], cv[UNR][SPL];
@@ -181,7 +181,7 @@ __device__ __forceinline__ float scan_walk(const float* __restrict__ dt_raw /* s
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
             const bool on = i + u < count;
-            const float step = on ? dt[u] : 0.f;
+            const float step = on ? (raw ? softplus_f32(dt[u]) : dt[u]) : 0.f;
             const float dx = step * xv[u];
             dt_sum += step;
             float y = 0.f;
@@ -256,7 +256,7 @@ __global__ void k_selective_scan(const float* __restrict__ dt_raw, const TX* __r
                                  const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len,
                                  const int32_t* __restrict__ slot, TOut* __restrict__ out,
                                  const float* __restrict__ scratch, int n_rows, int n_chunks, int channels, int n_state,
-                                 int lp) {
+                                 int lp, int raw) {
     const int r = blockIdx.x, k = blockIdx.z;
     const int len = seg_len[r];
     const int chunks = n_chunks > 1 ? max(1, (len + SCAN_CHUNK - 1) / SCAN_CHUNK) : 1;
@@ -288,7 +288,7 @@ __global__ void k_selective_scan(const float* __restrict__ dt_raw, const TX* __r
     const int first = chunks > 1 ? k * SCAN_CHUNK : 0;
     const int count = chunks > 1 ? min(SCAN_CHUNK, len - first) : len;
     scan_walk<TX, TOut, SPL, UNR, true>(dt_raw, x, bc, z, z_ld, out, S, a, D[cc], (size_t)seg_start[r] + first, count,
-                                        channels, cc, n_state, lp, ln, live);
+                                        channels, cc, n_state, lp, ln, live, raw != 0);
     if (live && k == chunks - 1 && len > 0) {
 #pragma unroll
         for (int j = 0; j < SPL; ++j) {
@@ -310,9 +310,13 @@ static int launch_scan(float* dt_raw, const void* x, const float* bc, const floa
     const int per_block = threads / lp;
     dim3 grid(n_rows, (channels + per_block - 1) / per_block, n_chunks);
     if (grid.y > 65535 || grid.z > 65535) return IMPARO_BAD_ARGUMENT;
-    const long long n_dt = (long long)n_tokens * channels;
-    k_softplus_rows<<<(unsigned)((n_dt + 255) / 256), 256, 0, s>>>(dt_raw, n_dt);
-    if (launch_status()) return IMPARO_LAUNCH_FAILED;
+    // one token a row (as many tokens as rows): softplus is taken inside the walk, a launch less for a decode step
+    const int raw = n_chunks == 1 && n_tokens == n_rows;
+    if (!raw) {
+        const long long n_dt = (long long)n_tokens * channels;
+        k_softplus_rows<<<(unsigned)((n_dt + 255) / 256), 256, 0, s>>>(dt_raw, n_dt);
+        if (launch_status()) return IMPARO_LAUNCH_FAILED;
+    }
 #define SCAN_LAUNCH(N, U)                                                                                             \
     do {                                                                                                              \
         if (n_chunks > 1) {                                                                                           \
@@ -323,7 +327,7 @@ static int launch_scan(float* dt_raw, const void* x, const float* bc, const floa
         }                                                                                                             \
         k_selective_scan<TX, TOut, N, U><<<grid, threads, 0, s>>>(dt_raw, (const TX*)x, bc, z, z_ld, A, D, state,     \
                                                                   seg_start, seg_len, slot, (TOut*)out, scratch,      \
-                                                                  n_rows, n_chunks, channels, n_state, lp);           \
+                                                                  n_rows, n_chunks, channels, n_state, lp, raw);      \
     } while (0)
     if (spl == 1 && lp >= 8) SCAN_LAUNCH(1, 8);        // a batch of tokens is finished by as many lanes of the channel
     else if (spl == 1 && lp == 4) SCAN_LAUNCH(1, 4);
@@ -338,7 +342,7 @@ static int launch_scan(float* dt_raw, const void* x, const float* bc, const floa
 }
 
 // dt_raw [tokens, channels] float32 (the step projection with its bias, before softplus; softplus is taken in
-// place, so the array holds the steps afterwards); x [tokens,
+// place, so the array holds the steps afterwards, unless every row brings one token: then inside the walk); x [tokens,
 // channels] in `dtype`; bc [tokens, 2 n_state] float32 (B then C); z rows z_ld floats apart; A, D float32
 // (A = -exp(A_log), [channels, n_state]); state [slots, channels, n_state] float32; out [tokens, channels]
 // in `dtype`. n_state at most 512. n_chunks 1: every segment is walked in one piece. More (at least

@@ -264,9 +264,11 @@ def attention_case(H, G, D, V, n_ctx, page, dtype, far=None, seed=0):
     return outs, ref
 
 
-@pytest.mark.parametrize("H,G,D,V,page", [(4, 2, 16, 32, 16), (3, 1, 24, 40, 64), (1, 1, 8, 8, 8), (2, 2, 20, 130, 32)])
+@pytest.mark.parametrize("H,G,D,V,page", [(4, 2, 16, 32, 16), (3, 1, 24, 40, 64), (1, 1, 8, 8, 8), (2, 2, 20, 130, 32),
+                                          (8, 1, 16, 96, 16), (8, 2, 36, 64, 32)])
 def test_differential_attention_kernel_float32(H, G, D, V, page):
-    """Every position of 700 keys over scrambled pages, whole and in splits of the keys."""
+    """Every position of 700 keys over scrambled pages, whole and in splits of the keys; one to eight heads
+    on a key/value head."""
     outs, ref = attention_case(H, G, D, V, 700, page, torch.float32, seed=H)
     for n_splits, out in outs.items():
         assert torch.allclose(out, ref, atol=2e-5, rtol=1e-4), f"{n_splits} splits: {float((out - ref).abs().max())}"
