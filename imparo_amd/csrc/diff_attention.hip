@@ -266,30 +266,46 @@ __global__ void k_diff_merge(const float* __restrict__ part, const float* __rest
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
     const int s_first = lo / DA_SPLIT, s_last = min(pos / DA_SPLIT, n_splits - 1);
     const float* base = part + (size_t)th * n_splits * (2 * vdim + 4);
+    const int stride = 2 * vdim + 4;
+    // the splits' maxima: a split a lane, 64 at a time
     float m1 = -INFINITY, m2 = -INFINITY;
-    for (int s = s_first; s <= s_last; ++s) {
-        const float* p = base + (size_t)s * (2 * vdim + 4);
-        m1 = fmaxf(m1, p[0]);
-        m2 = fmaxf(m2, p[2]);
+    for (int s0 = s_first; s0 <= s_last; s0 += WAVE) {
+        const int s = min(s0 + lane, s_last);
+        m1 = fmaxf(m1, base[(size_t)s * stride]);
+        m2 = fmaxf(m2, base[(size_t)s * stride + 2]);
     }
+    m1 = wave_max(m1);
+    m2 = wave_max(m2);
     float a1[VPL], a2[VPL];
 #pragma unroll
     for (int j = 0; j < VPL; ++j) a1[j] = a2[j] = 0.f;
     float l1 = 0.f, l2 = 0.f;
-    for (int s = s_first; s <= s_last; ++s) {
-        const float* p = base + (size_t)s * (2 * vdim + 4);
-        const float w1 = p[0] == -INFINITY ? 0.f : expf(p[0] - m1);
-        const float w2 = p[2] == -INFINITY ? 0.f : expf(p[2] - m2);
-        l1 += w1 * p[1];
-        l2 += w2 * p[3];
+    // the weighted sums in the order of the splits, four splits' rows asked for at once
+    for (int s0 = s_first; s0 <= s_last; s0 += 4) {
+        float w1[4], w2[4], r1[4][VPL], r2[4][VPL];
 #pragma unroll
-        for (int j = 0; j < VPL; ++j) {
-            const int d = lane + j * WAVE;
-            if (d < vdim) {
-                a1[j] += w1 * p[4 + d];
-                a2[j] += w2 * p[4 + vdim + d];
+        for (int u = 0; u < 4; ++u) {
+            const bool on = s0 + u <= s_last;
+            const float* p = base + (size_t)min(s0 + u, s_last) * stride;
+            const float pm1 = p[0], pl1 = p[1], pm2 = p[2], pl2 = p[3];
+            w1[u] = on && pm1 != -INFINITY ? expf(pm1 - m1) : 0.f;
+            w2[u] = on && pm2 != -INFINITY ? expf(pm2 - m2) : 0.f;
+            l1 += w1[u] * pl1;
+            l2 += w2[u] * pl2;
+#pragma unroll
+            for (int j = 0; j < VPL; ++j) {
+                const int d = min(lane + j * WAVE, vdim - 1);
+                r1[u][j] = p[4 + d];
+                r2[u][j] = p[4 + vdim + d];
             }
         }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int j = 0; j < VPL; ++j) {
+                a1[j] += w1[u] * r1[u][j];
+                a2[j] += w2[u] * r2[u][j];
+            }
     }
     const float i1 = l1 > 0.f ? 1.0f / l1 : 0.f, i2 = l2 > 0.f ? 1.0f / l2 : 0.f;
 #pragma unroll
@@ -380,6 +396,7 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
     const int pos_first = positions[t0 + q0], pos_last = positions[t0 + q0 + n_q - 1];
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
     const int lo_first = window > 0 ? max(0, pos_first + 1 - window) : 0;
+    const int lo_last = window > 0 ? max(0, pos_last + 1 - window) : 0;
     const int g = h / (heads / kv_heads);
     const int vd16 = (vdim + 15) >> 4;
     const int32_t* table = block_table + (size_t)r * table_stride;
@@ -424,6 +441,8 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
 
         da_s16x4 pb[2][2];                                   // P^T operands: [map][block of 16 keys]
         float corr[2];
+        // a tile that every query of the wave sees whole needs no look at single keys (uniform over the wave)
+        const bool whole = cur.there[0] && cur.there[1] && k0 + 31 <= pos_first && k0 >= lo_last;
 #pragma unroll
         for (int m = 0; m < 2; ++m) {
             da_f32x4 sc[2] = {da_f32x4{0.f, 0.f, 0.f, 0.f}, da_f32x4{0.f, 0.f, 0.f, 0.f}};
@@ -434,15 +453,25 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
                     sc[mb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(cur.k[m][mb][kk], qf[m][kk], sc[mb], 0, 0, 0);
             // a lane holds keys k0 + 16 mb + 4 quad + i of query `col`
             float tile_max = -INFINITY;
+            if (whole) {
 #pragma unroll
-            for (int mb = 0; mb < 2; ++mb)
+                for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int key = k0 + mb * 16 + quad * 4 + i;
-                    const bool seen = cur.there[mb] && key <= pos && key >= lo;
-                    sc[mb][i] = seen ? sc[mb][i] * scale : -INFINITY;
-                    tile_max = fmaxf(tile_max, sc[mb][i]);
-                }
+                    for (int i = 0; i < 4; ++i) {
+                        sc[mb][i] *= scale;
+                        tile_max = fmaxf(tile_max, sc[mb][i]);
+                    }
+            } else {
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = k0 + mb * 16 + quad * 4 + i;
+                        const bool seen = cur.there[mb] && key <= pos && key >= lo;
+                        sc[mb][i] = seen ? sc[mb][i] * scale : -INFINITY;
+                        tile_max = fmaxf(tile_max, sc[mb][i]);
+                    }
+            }
             tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
             tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
             const float m_new = fmaxf(mx[m], tile_max);
@@ -464,25 +493,32 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb) pb[m][mb] = da_pack4(p[mb][0], p[mb][1], p[mb][2], p[mb][3]);
         }
+        // the old sums are rescaled only when some query's maximum moved (uniform over the wave)
+        const bool rescale = __any(corr[0] != 1.0f || corr[1] != 1.0f);
 #pragma unroll
         for (int vb = 0; vb < V16; ++vb) {
             if (vb < vd16) {
+                if (rescale) {
 #pragma unroll
-                for (int m = 0; m < 2; ++m) {
-                    o[m][vb][0] *= corr[m];
-                    o[m][vb][1] *= corr[m];
-                    o[m][vb][2] *= corr[m];
-                    o[m][vb][3] *= corr[m];
+                    for (int m = 0; m < 2; ++m) {
+                        o[m][vb][0] *= corr[m];
+                        o[m][vb][1] *= corr[m];
+                        o[m][vb][2] *= corr[m];
+                        o[m][vb][3] *= corr[m];
+                    }
                 }
                 const bool on_d = vb * 16 + col < vdim;
 #pragma unroll
                 for (int mb = 0; mb < 2; ++mb) {
                     da_s16x4 v = vt[mb][vb];
-                    const int key = k0 + mb * 16 + quad * 4;         // what lies past the last query's position is not a value yet
-                    if (key + 1 > pos_last) v[1] = 0;
-                    if (key + 2 > pos_last) v[2] = 0;
-                    if (key + 3 > pos_last) v[3] = 0;
-                    if (!(on_d && cur.there[mb]) || key > pos_last) v = da_s16x4{0, 0, 0, 0};
+                    if (!whole) {
+                        const int key = k0 + mb * 16 + quad * 4;     // what lies past the last query's position is not a value yet
+                        if (key + 1 > pos_last) v[1] = 0;
+                        if (key + 2 > pos_last) v[2] = 0;
+                        if (key + 3 > pos_last) v[3] = 0;
+                        if (!cur.there[mb] || key > pos_last) v = da_s16x4{0, 0, 0, 0};
+                    }
+                    if (!on_d) v = da_s16x4{0, 0, 0, 0};
                     o[0][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v, pb[0][mb], o[0][vb], 0, 0, 0);
                     o[1][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v, pb[1][mb], o[1][vb], 0, 0, 0);
                 }
