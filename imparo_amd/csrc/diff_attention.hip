@@ -562,6 +562,261 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
     }
 }
 
+// The same walk with every tile staged once a block: the four waves of a block (64 consecutive queries
+// of one head) walk the same keys, so each tile of 32 keys is brought into LDS by all 256 threads
+// together, K rows as they lie (rows 8 bytes apart from a power of two, so that the operand reads of 16
+// rows spread over the banks) and V transposed on the way in, [value dimension][key], so that the second
+// product's operand, four consecutive keys of one value dimension, is one 8-byte read. The next tile's
+// global loads are in flight in registers while this tile's products run. For dim and vdim multiples of 8.
+#define DAS_KPAD 4           // bf16 elements between K rows in LDS beyond dim
+#define DAS_VROW 36          // bf16 elements of a V^T row in LDS: 32 keys + 4
+
+template <int D16, int V16>
+__global__ __launch_bounds__(256) void k_diff_attention_shared(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const float* __restrict__ gate, int gate_ld, bf16_t* __restrict__ out, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len,
+    const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int dim,
+    int vdim, int n_pages, float scale, int window, float lambda, float eps, float out_scale, int min_len) {
+    __shared__ __attribute__((aligned(16))) bf16_t k_lds[2 * 32 * (16 * D16 + DAS_KPAD)];
+    __shared__ __attribute__((aligned(16))) bf16_t v_lds[16 * V16 * DAS_VROW];
+    const int r = blockIdx.x, h = blockIdx.z;
+    const int len = seg_len[r];
+    if (len < min_len) return;                                 // (uniform over the block)
+    const int b0 = blockIdx.y * DAM_TILE;                      // the block's first query within the portion
+    if (b0 >= len) return;                                     // (uniform over the block)
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int col = lane & 15, quad = lane >> 4;
+    const int t0 = seg_start[r];
+    const int q0 = b0 + wave * 16;
+    const bool wave_on = q0 < len;                             // a wave past the portion helps to stage and computes nothing
+    const int n_q = wave_on ? min(16, len - q0) : 1;
+    const int qi = wave_on ? min(col, n_q - 1) : 0;
+    const int t = t0 + (wave_on ? q0 + qi : b0);
+    const int pos = positions[t];
+    const int pos_first = positions[t0 + (wave_on ? q0 : b0)], pos_last = positions[t0 + (wave_on ? q0 + n_q - 1 : b0)];
+    const int block_first = positions[t0 + b0], block_last = positions[t0 + min(b0 + DAM_TILE, len) - 1];
+    const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    const int lo_first = window > 0 ? max(0, pos_first + 1 - window) : 0;
+    const int lo_last = window > 0 ? max(0, pos_last + 1 - window) : 0;
+    const int lo_block = window > 0 ? max(0, block_first + 1 - window) : 0;
+    const int g = h / (heads / kv_heads);
+    const int vd16 = (vdim + 15) >> 4;
+    const int krow = dim + DAS_KPAD;
+    const int32_t* table = block_table + (size_t)r * table_stride;
+
+    da_s16x4 qf[2][D16];
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int kk = 0; kk < D16; ++kk) {
+            const int d = kk * 16 + quad * 4;
+            const da_s16x4 v = *reinterpret_cast<const da_s16x4*>(q + (((size_t)t * heads + h) * 2 + m) * dim + min(d, dim - 4));
+            qf[m][kk] = d < dim ? v : da_s16x4{0, 0, 0, 0};
+        }
+    da_f32x4 o[2][V16];
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int vb = 0; vb < V16; ++vb) o[m][vb] = da_f32x4{0.f, 0.f, 0.f, 0.f};
+    float mx[2] = {-INFINITY, -INFINITY}, sum[2] = {0.f, 0.f};
+
+    // staging: a thread's 16-byte pieces of the K tile (64 rows: map, key) and of the V tile (32 rows: key)
+    constexpr int KP = (2 * 32 * 2 * D16 + 255) / 256;         // pieces of 8 elements a thread, K: 64 rows x dim / 8
+    constexpr int VP = (32 * 2 * V16 + 255) / 256;             // V: 32 rows x vdim / 8
+    const int k_per_row = dim >> 3, v_per_row = vdim >> 3;
+    uint4 kreg[KP], vreg[VP];
+    auto ask = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            const int c = threadIdx.x + i * 256;
+            const int row = min(c / k_per_row, 63), part = c - (c / k_per_row) * k_per_row;
+            const int m = row >> 5, key = row & 31;
+            const int key0 = k0 + (key & 16);
+            const int page = key0 <= block_last ? table[key0 / page_size] : -1;
+            const bool on = page >= 0 && page < n_pages && c < 64 * k_per_row;
+            const long long pg = on ? page : 0;
+            const uint4 v = *reinterpret_cast<const uint4*>(
+                k_cache + ((pg * 2 * kv_heads + 2 * g + m) * page_size + ((k0 + key) % page_size)) * dim + part * 8);
+            kreg[i] = on ? v : uint4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const int c = threadIdx.x + i * 256;
+            const int key = min(c / v_per_row, 31), part = c - (c / v_per_row) * v_per_row;
+            const int key0 = k0 + (key & 16);
+            const int page = key0 <= block_last ? table[key0 / page_size] : -1;
+            // what lies past the block's last position is not a value yet: zeros, which weigh nothing
+            const bool on = page >= 0 && page < n_pages && c < 32 * v_per_row && k0 + key <= block_last;
+            const long long pg = on ? page : 0;
+            const uint4 v = *reinterpret_cast<const uint4*>(
+                v_cache + ((pg * kv_heads + g) * page_size + ((k0 + key) % page_size)) * (long long)vdim + part * 8);
+            vreg[i] = on ? v : uint4{0, 0, 0, 0};
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            const int c = threadIdx.x + i * 256;
+            if (c < 64 * k_per_row) {
+                const int row = c / k_per_row, part = c - row * k_per_row;
+                // rows lie krow elements apart: 8 bytes past a multiple of 16, so a piece goes in two halves
+                uint2* dst = reinterpret_cast<uint2*>(k_lds + row * krow + part * 8);
+                dst[0] = uint2{kreg[i].x, kreg[i].y};
+                dst[1] = uint2{kreg[i].z, kreg[i].w};
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const int c = threadIdx.x + i * 256;
+            if (c < 32 * v_per_row) {
+                const int key = c / v_per_row, part = c - key * v_per_row;
+                const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v_lds[(part * 8 + 2 * e) * DAS_VROW + key] = (bf16_t)(w[e] & 0xffff);
+                    v_lds[(part * 8 + 2 * e + 1) * DAS_VROW + key] = (bf16_t)(w[e] >> 16);
+                }
+            }
+        }
+    };
+
+    int k0 = (lo_block / 32) * 32;
+    ask(k0);
+    stage();
+    __syncthreads();
+    for (; k0 <= block_last; k0 += 32) {
+        if (k0 + 32 <= block_last) ask(k0 + 32);               // (uniform over the block)
+        if (wave_on && k0 <= pos_last && k0 + 31 >= lo_first) {
+            da_s16x4 pb[2][2];
+            float corr[2];
+            bool there[2];
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) {
+                const int key0 = k0 + mb * 16;
+                const int page = key0 <= pos_last ? table[key0 / page_size] : -1;
+                there[mb] = page >= 0 && page < n_pages;
+            }
+            const bool whole = there[0] && there[1] && k0 + 31 <= pos_first && k0 >= lo_last;
+#pragma unroll
+            for (int m = 0; m < 2; ++m) {
+                da_f32x4 sc[2] = {da_f32x4{0.f, 0.f, 0.f, 0.f}, da_f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                    for (int kk = 0; kk < D16; ++kk) {
+                        const int d = min(kk * 16 + quad * 4, dim - 4);
+                        const da_s16x4 kf = *reinterpret_cast<const da_s16x4*>(k_lds + (m * 32 + mb * 16 + col) * krow + d);
+                        sc[mb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf, qf[m][kk], sc[mb], 0, 0, 0);
+                    }
+                float tile_max = -INFINITY;
+                if (whole) {
+#pragma unroll
+                    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            sc[mb][i] *= scale;
+                            tile_max = fmaxf(tile_max, sc[mb][i]);
+                        }
+                } else {
+#pragma unroll
+                    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int key = k0 + mb * 16 + quad * 4 + i;
+                            const bool seen = there[mb] && key <= pos && key >= lo;
+                            sc[mb][i] = seen ? sc[mb][i] * scale : -INFINITY;
+                            tile_max = fmaxf(tile_max, sc[mb][i]);
+                        }
+                }
+                tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
+                tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
+                const float m_new = fmaxf(mx[m], tile_max);
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                corr[m] = mx[m] == -INFINITY ? 0.f : __expf(mx[m] - m_use);
+                float tile_sum = 0.f;
+                float p[2][4];
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        p[mb][i] = __expf(sc[mb][i] - m_use);
+                        tile_sum += p[mb][i];
+                    }
+                tile_sum += __shfl_xor(tile_sum, 16, WAVE);
+                tile_sum += __shfl_xor(tile_sum, 32, WAVE);
+                sum[m] = sum[m] * corr[m] + tile_sum;
+                mx[m] = m_new;
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb) pb[m][mb] = da_pack4(p[mb][0], p[mb][1], p[mb][2], p[mb][3]);
+            }
+            const bool rescale = __any(corr[0] != 1.0f || corr[1] != 1.0f);
+#pragma unroll
+            for (int vb = 0; vb < V16; ++vb) {
+                if (vb < vd16) {
+                    if (rescale) {
+#pragma unroll
+                        for (int m = 0; m < 2; ++m) {
+                            o[m][vb][0] *= corr[m];
+                            o[m][vb][1] *= corr[m];
+                            o[m][vb][2] *= corr[m];
+                            o[m][vb][3] *= corr[m];
+                        }
+                    }
+                    const int d = min(vb * 16 + col, vdim - 1);
+                    const bool on_d = vb * 16 + col < vdim;
+#pragma unroll
+                    for (int mb = 0; mb < 2; ++mb) {
+                        // keys 4 quad .. + 3 of the block, value dimension d: eight bytes of a V^T row. A key that this
+                        // wave's queries do not see weighs nothing (its P is zero) and its value is finite or zero
+                        da_s16x4 v = *reinterpret_cast<const da_s16x4*>(v_lds + d * DAS_VROW + mb * 16 + quad * 4);
+                        if (!on_d) v = da_s16x4{0, 0, 0, 0};
+                        o[0][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v, pb[0][mb], o[0][vb], 0, 0, 0);
+                        o[1][vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v, pb[1][mb], o[1][vb], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        __syncthreads();                                       // every wave has read this tile
+        if (k0 + 32 <= block_last) stage();
+        __syncthreads();
+    }
+    if (!wave_on) return;
+    const float i1 = sum[0] > 0.f ? 1.0f / sum[0] : 0.f, i2 = sum[1] > 0.f ? 1.0f / sum[1] : 0.f;
+    float ss = 0.f;
+#pragma unroll
+    for (int vb = 0; vb < V16; ++vb)
+        if (vb < vd16) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool on = vb * 16 + quad * 4 + i < vdim;
+                const float v = on ? o[0][vb][i] * i1 - lambda * (o[1][vb][i] * i2) : 0.f;
+                o[0][vb][i] = v;
+                ss += v * v;
+            }
+        }
+    ss += __shfl_xor(ss, 16, WAVE);
+    ss += __shfl_xor(ss, 32, WAVE);
+    const float rr = out_scale / sqrtf(ss / (float)vdim + eps);
+    if (col < n_q) {
+        const float* gt = gate ? gate + (size_t)t * gate_ld + (size_t)h * vdim : nullptr;
+        bf16_t* dst = out + ((size_t)t * heads + h) * vdim;
+#pragma unroll
+        for (int vb = 0; vb < V16; ++vb)
+            if (vb < vd16) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int d = vb * 16 + quad * 4 + i;
+                    if (d < vdim) {
+                        float y = o[0][vb][i] * rr;
+                        if (gt) y *= 1.0f / (1.0f + __expf(-gt[d]));
+                        dst[d] = f32_to_bf16(y);
+                    }
+                }
+            }
+    }
+}
+
 // Whether the matrix-core kernel takes these sizes (bfloat16 only).
 extern "C" int imparo_diff_attention_tiles_takes(int page_size, int dim, int vdim) {
     return page_size >= 16 && page_size % 16 == 0 && dim > 0 && vdim > 0 && dim % 4 == 0 && vdim % 4 == 0 &&
@@ -590,10 +845,21 @@ extern "C" int imparo_diff_attention_tiles(const void* q, const void* k_cache, c
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, gate, gate_ld, (bf16_t*)out, positions, seg_start, \
         seg_len, block_table, table_stride, page_size, heads, kv_heads, dim, vdim, n_pages, scale, window, lambda, eps,   \
         out_scale, min_len)
-    if (dim <= 64 && vdim <= 64) DAM_LAUNCH(4, 4);
+#define DAS_LAUNCH(D16, V16)                                                                                             \
+    k_diff_attention_shared<D16, V16><<<grid, 256, 0, (hipStream_t)stream>>>(                                             \
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, gate, gate_ld, (bf16_t*)out, positions, seg_start, \
+        seg_len, block_table, table_stride, page_size, heads, kv_heads, dim, vdim, n_pages, scale, window, lambda, eps,   \
+        out_scale, min_len)
+    if (dim % 8 == 0 && vdim % 8 == 0) {          // every tile staged once a block in LDS
+        if (dim <= 64 && vdim <= 64) DAS_LAUNCH(4, 4);
+        else if (dim <= 64) DAS_LAUNCH(4, 8);
+        else if (vdim <= 64) DAS_LAUNCH(8, 4);
+        else DAS_LAUNCH(8, 8);
+    } else if (dim <= 64 && vdim <= 64) DAM_LAUNCH(4, 4);
     else if (dim <= 64) DAM_LAUNCH(4, 8);
     else if (vdim <= 64) DAM_LAUNCH(8, 4);
     else DAM_LAUNCH(8, 8);
+#undef DAS_LAUNCH
 #undef DAM_LAUNCH
     return launch_status();
 }
