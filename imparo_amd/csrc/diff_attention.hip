@@ -583,7 +583,8 @@ __global__ __launch_bounds__(256) void k_diff_attention_shared(
     const int r = blockIdx.x, h = blockIdx.z;
     const int len = seg_len[r];
     if (len < min_len) return;                                 // (uniform over the block)
-    const int b0 = blockIdx.y * DAM_TILE;                      // the block's first query within the portion
+    // the last queries walk the most keys: their blocks go first (blocks start in the order of their numbers)
+    const int b0 = ((int)gridDim.y - 1 - (int)blockIdx.y) * DAM_TILE;     // the block's first query within the portion
     if (b0 >= len) return;                                     // (uniform over the block)
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int col = lane & 15, quad = lane >> 4;
@@ -603,6 +604,7 @@ __global__ __launch_bounds__(256) void k_diff_attention_shared(
     const int g = h / (heads / kv_heads);
     const int vd16 = (vdim + 15) >> 4;
     const int krow = dim + DAS_KPAD;
+    const int page_shift = __ffs(page_size) - 1, page_mask = page_size - 1;     // pages are a power of two
     const int32_t* table = block_table + (size_t)r * table_stride;
 
     da_s16x4 qf[2][D16];
@@ -626,56 +628,67 @@ __global__ __launch_bounds__(256) void k_diff_attention_shared(
     constexpr int VP = (32 * 2 * V16 + 255) / 256;             // V: 32 rows x vdim / 8
     const int k_per_row = dim >> 3, v_per_row = vdim >> 3;
     uint4 kreg[KP], vreg[VP];
+    // which piece of a tile a thread brings does not change from tile to tile
+    int k_row[KP], k_part[KP], v_key[VP], v_part[VP];
+    bool k_in[KP], v_in[VP];
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+        const int c = threadIdx.x + i * 256;
+        k_in[i] = c < 64 * k_per_row;
+        k_row[i] = min(c / k_per_row, 63);
+        k_part[i] = c - (c / k_per_row) * k_per_row;
+    }
+#pragma unroll
+    for (int i = 0; i < VP; ++i) {
+        const int c = threadIdx.x + i * 256;
+        v_in[i] = c < 32 * v_per_row;
+        v_key[i] = min(c / v_per_row, 31);
+        v_part[i] = c - (c / v_per_row) * v_per_row;
+    }
     auto ask = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < KP; ++i) {
-            const int c = threadIdx.x + i * 256;
-            const int row = min(c / k_per_row, 63), part = c - (c / k_per_row) * k_per_row;
-            const int m = row >> 5, key = row & 31;
+            const int m = k_row[i] >> 5, key = k_row[i] & 31;
             const int key0 = k0 + (key & 16);
-            const int page = key0 <= block_last ? table[key0 / page_size] : -1;
-            const bool on = page >= 0 && page < n_pages && c < 64 * k_per_row;
+            const int page = key0 <= block_last ? table[key0 >> page_shift] : -1;
+            const bool on = page >= 0 && page < n_pages && k_in[i];
             const long long pg = on ? page : 0;
             const uint4 v = *reinterpret_cast<const uint4*>(
-                k_cache + ((pg * 2 * kv_heads + 2 * g + m) * page_size + ((k0 + key) % page_size)) * dim + part * 8);
+                k_cache + ((pg * 2 * kv_heads + 2 * g + m) * page_size + ((k0 + key) & page_mask)) * dim + k_part[i] * 8);
             kreg[i] = on ? v : uint4{0, 0, 0, 0};
         }
 #pragma unroll
         for (int i = 0; i < VP; ++i) {
-            const int c = threadIdx.x + i * 256;
-            const int key = min(c / v_per_row, 31), part = c - (c / v_per_row) * v_per_row;
+            const int key = v_key[i];
             const int key0 = k0 + (key & 16);
-            const int page = key0 <= block_last ? table[key0 / page_size] : -1;
+            const int page = key0 <= block_last ? table[key0 >> page_shift] : -1;
             // what lies past the block's last position is not a value yet: zeros, which weigh nothing
-            const bool on = page >= 0 && page < n_pages && c < 32 * v_per_row && k0 + key <= block_last;
+            const bool on = page >= 0 && page < n_pages && v_in[i] && k0 + key <= block_last;
             const long long pg = on ? page : 0;
             const uint4 v = *reinterpret_cast<const uint4*>(
-                v_cache + ((pg * kv_heads + g) * page_size + ((k0 + key) % page_size)) * (long long)vdim + part * 8);
+                v_cache + ((pg * kv_heads + g) * page_size + ((k0 + key) & page_mask)) * (long long)vdim + v_part[i] * 8);
             vreg[i] = on ? v : uint4{0, 0, 0, 0};
         }
     };
     auto stage = [&]() {
 #pragma unroll
         for (int i = 0; i < KP; ++i) {
-            const int c = threadIdx.x + i * 256;
-            if (c < 64 * k_per_row) {
-                const int row = c / k_per_row, part = c - row * k_per_row;
+            if (k_in[i]) {
                 // rows lie krow elements apart: 8 bytes past a multiple of 16, so a piece goes in two halves
-                uint2* dst = reinterpret_cast<uint2*>(k_lds + row * krow + part * 8);
+                uint2* dst = reinterpret_cast<uint2*>(k_lds + k_row[i] * krow + k_part[i] * 8);
                 dst[0] = uint2{kreg[i].x, kreg[i].y};
                 dst[1] = uint2{kreg[i].z, kreg[i].w};
             }
         }
 #pragma unroll
         for (int i = 0; i < VP; ++i) {
-            const int c = threadIdx.x + i * 256;
-            if (c < 32 * v_per_row) {
-                const int key = c / v_per_row, part = c - key * v_per_row;
+            if (v_in[i]) {
                 const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+                bf16_t* dst = v_lds + (v_part[i] * 8) * DAS_VROW + v_key[i];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    v_lds[(part * 8 + 2 * e) * DAS_VROW + key] = (bf16_t)(w[e] & 0xffff);
-                    v_lds[(part * 8 + 2 * e + 1) * DAS_VROW + key] = (bf16_t)(w[e] >> 16);
+                    dst[(2 * e) * DAS_VROW] = (bf16_t)(w[e] & 0xffff);
+                    dst[(2 * e + 1) * DAS_VROW] = (bf16_t)(w[e] >> 16);
                 }
             }
         }
@@ -694,7 +707,7 @@ __global__ __launch_bounds__(256) void k_diff_attention_shared(
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb) {
                 const int key0 = k0 + mb * 16;
-                const int page = key0 <= pos_last ? table[key0 / page_size] : -1;
+                const int page = key0 <= pos_last ? table[key0 >> page_shift] : -1;
                 there[mb] = page >= 0 && page < n_pages;
             }
             const bool whole = there[0] && there[1] && k0 + 31 <= pos_first && k0 >= lo_last;
@@ -850,7 +863,7 @@ extern "C" int imparo_diff_attention_tiles(const void* q, const void* k_cache, c
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, gate, gate_ld, (bf16_t*)out, positions, seg_start, \
         seg_len, block_table, table_stride, page_size, heads, kv_heads, dim, vdim, n_pages, scale, window, lambda, eps,   \
         out_scale, min_len)
-    if (dim % 8 == 0 && vdim % 8 == 0) {          // every tile staged once a block in LDS
+    if (dim % 8 == 0 && vdim % 8 == 0 && (page_size & (page_size - 1)) == 0) {          // every tile staged once a block in LDS
         if (dim <= 64 && vdim <= 64) DAS_LAUNCH(4, 4);
         else if (dim <= 64) DAS_LAUNCH(4, 8);
         else if (vdim <= 64) DAS_LAUNCH(8, 4);
