@@ -572,7 +572,7 @@ __global__ __launch_bounds__(256) void k_diff_attention_tiles(
 #define DAS_VROW 36          // bf16 elements of a V^T row in LDS: 32 keys + 4
 
 template <int D16, int V16>
-__global__ __launch_bounds__(256) void k_diff_attention_shared(
+__global__ __launch_bounds__(256, 2) void k_diff_attention_shared(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const float* __restrict__ gate, int gate_ld, bf16_t* __restrict__ out, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len,
