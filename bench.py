@@ -393,11 +393,11 @@ def tumadra_shape(width, heads, kv_heads, ff, inner, layers=16, attention_at=(2,
     they have attention (two maps of 64 a head, values of 128: the same q, k, v and output widths as their
     heads of 64), a selective scan where they have a short conv (inner chosen so that the mixer's matrices
     weigh what the conv block's do), a dense PolyNorm feed-forward with the parameters of their SwiGLU."""
-    attention = dict(heads=heads, kv_heads=kv_heads, dim=64, vdim=128, scale=0.125, diff=0.6,
-                     q_temp=dict(coef=0.3, every=256))
+    attention = dict(heads=heads, kv_heads=kv_heads, dim=64, vdim=128, scale=0.125, diff=0.5,
+                     q_temp=dict(coef=0.25, every=512))
     scan = dict(inner=inner, state=16, dt_rank=width // 16, conv=4)
     mlp = dict(kind="dense", ff=ff)
-    return dict(architecture="Tumadra", vocab=65536, width=width, norm=dict(eps=1e-5, groups=4),
+    return dict(architecture="Tumadra", vocab=65536, width=width, norm=dict(eps=1e-6, groups=8),
                 layers=[dict(type="attention" if i in attention_at else "mamba1",
                              mixer=attention if i in attention_at else scan, mlp=mlp) for i in range(layers)])
 
