@@ -25,7 +25,7 @@ from ..config.plan import PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .base import Declared, StepContext
-from .linear import Linear, place_matrix
+from .linear import Linear, place_matrix, place_projection
 from .registry import register_part
 
 _DEFAULT_NAMES = dict(q="q", k="k", v="v", g="g", o="o", lq1="lq1", lk1="lk1", lq2="lq2", lk2="lk2", bias="b")
@@ -91,8 +91,11 @@ class DifferentialAttention:
                 bs.append(torch.zeros(self.heads * self.vdim))
             bias = torch.cat(bs).to(device)
         # one projection for q | k | v | gate logits: the same dot products, one launch
-        self.qkvg = Linear(place_matrix(torch.cat(ws, dim=0), engine_dtype, device), bias)
+        self.qkvg = Linear(place_projection(torch.cat(ws, dim=0), engine_dtype, device), bias)
         self.gate_at = (self.heads + self.kv_heads) * 2 * self.dim + self.kv_heads * self.vdim
+        if engine_dtype != torch.float32 and (self.heads * self.vdim) % 8:
+            raise ValueError(f"under bfloat16 the output projection walks its {self.heads} x {self.vdim} inputs in steps "
+                             f"of 8; run this model with dtype float32")
         self.out = Linear(place_matrix(tensors[n["o"]], engine_dtype, device))
         l = {x: tensors[n[x]].to(torch.float32) for x in ("lq1", "lk1", "lq2", "lk2")}
         self.lam = float(torch.exp((l["lq1"] * l["lk1"]).sum()) - torch.exp((l["lq2"] * l["lk2"]).sum())) + self.diff

@@ -18,7 +18,7 @@ from ..config.plan import PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .base import Declared, StepContext
-from .linear import Linear, place_matrix
+from .linear import Linear, place_matrix, place_projection
 from .registry import register_part
 
 
@@ -79,7 +79,7 @@ class LinearHead:
                  engine_dtype: torch.dtype, placed: Dict[str, torch.Tensor]):
         name = _table_name(spec)
         if name not in placed:
-            placed[name] = place_matrix(tensors[name], engine_dtype, device)
+            placed[name] = place_projection(tensors[name], engine_dtype, device)
         self.proj = Linear(placed[name])
         self.vocab = spec["vocab"]
 

@@ -15,7 +15,7 @@ from ..config.plan import PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .base import Declared, StepContext
-from .linear import Linear, place_matrix, place_vector
+from .linear import Linear, place_matrix, place_projection, place_vector
 from .registry import register_part
 
 _DEFAULT_NAMES = dict(gate="gate_proj", up="up_proj", down="down_proj")
@@ -112,7 +112,7 @@ class PolyNormFfn:
         if fill and engine_dtype != torch.float32 and down.dtype != torch.float32:
             up = torch.cat([up, up.new_zeros(fill, self.width)])
             down = torch.cat([down, down.new_zeros(self.width, fill)], dim=1)
-        self.up = Linear(place_matrix(up, engine_dtype, device))
+        self.up = Linear(place_projection(up, engine_dtype, device))
         self.down = Linear(place_matrix(down, engine_dtype, device))
         self.coef = place_vector(tensors[n["act"]], device)
 

@@ -62,6 +62,16 @@ def place_matrix(t: torch.Tensor, engine_dtype: torch.dtype, device: torch.devic
     return t.to(device=device, dtype=torch.bfloat16).contiguous()
 
 
+def place_projection(t: torch.Tensor, engine_dtype: torch.dtype, device: torch.device) -> torch.Tensor:
+    """`place_matrix` for a projection weight [out, in] whose inner size any model may choose: the
+    bfloat16 kernels walk the inner size in steps of 8, so a weight over another inner size is kept in
+    float32 and its projection runs the float32 kernel (whoever makes its input is asked for float32
+    through `in_dtype`)."""
+    if engine_dtype != torch.float32 and t.dim() == 2 and t.shape[1] % 8:
+        t = t.to(torch.float32)
+    return place_matrix(t, engine_dtype, device)
+
+
 def place_vector(t: torch.Tensor, device: torch.device) -> torch.Tensor:
     """Norm weights, conv taps and biases are read as float32 by the kernels;
     widening bfloat16 to float32 is exact."""

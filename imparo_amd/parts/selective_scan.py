@@ -19,7 +19,7 @@ from ..config.plan import PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .base import Declared, StepContext
-from .linear import Linear, place_matrix, place_vector
+from .linear import Linear, place_matrix, place_projection, place_vector
 from .registry import register_part
 
 _DEFAULT_NAMES = {"in": "in", "conv": "conv", "conv_bias": "conv.b", "x": "x", "dt": "dt", "dt_bias": "dt.b",
@@ -62,12 +62,14 @@ class SelectiveScan:
         if self.n_state > 512:
             raise ValueError(f"the scan kernel takes up to 512 states a channel, got {self.n_state}")
         R, N = self.dt_rank, self.n_state
-        self.in_proj = Linear(place_matrix(tensors[n["in"]], engine_dtype, device))
+        self.in_proj = Linear(place_projection(tensors[n["in"]], engine_dtype, device))
         wx, wdt = tensors[n["x"]], tensors[n["dt"]]
         if wx.dtype != wdt.dtype:
             wx, wdt = wx.to(torch.float32), wdt.to(torch.float32)
         # The step's low-rank input is a product's inner size, which the bfloat16 kernels walk in steps of 8:
         # it is filled up with units of zero weight on both sides, which add nothing to any sum.
+        if engine_dtype != torch.float32 and self.inner % 8:
+            wx, wdt = wx.to(torch.float32), wdt.to(torch.float32)      # the scan's side of the mixer in float32 then
         fill = (-R) % 8 if (engine_dtype != torch.float32 and wx.dtype != torch.float32) else 0
         low, step = wx[:R], wdt
         if fill:
@@ -77,7 +79,7 @@ class SelectiveScan:
         self.x_low = Linear(place_matrix(low, engine_dtype, device))
         self.x_bc = Linear(place_matrix(wx[R:], engine_dtype, device))
         self.dt_proj = Linear(place_matrix(step, engine_dtype, device), place_vector(tensors[n["dt_bias"]], device))
-        self.out_proj = Linear(place_matrix(tensors[n["o"]], engine_dtype, device))
+        self.out_proj = Linear(place_projection(tensors[n["o"]], engine_dtype, device))
         self.conv_weight = place_vector(tensors[n["conv"]].reshape(self.inner, self.taps), device)
         self.conv_bias = place_vector(tensors[n["conv_bias"]], device)
         self.A = (-torch.exp(tensors[n["A_log"]].to(torch.float32))).to(device).contiguous()

@@ -340,7 +340,7 @@ def test_differential_attention_matrix_core_kernel(H, G, D, V, page):
 
 # ------------------------------------------------------------------ the model in the engine
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_whole_prompt_and_stepwise(dirs, plains, name, dtype):
     """A prompt whole; then most of it whole and its last 40 tokens one by one (captured steps)."""
     from imparo_amd.engine import StepEntry
@@ -361,7 +361,7 @@ def test_whole_prompt_and_stepwise(dirs, plains, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,page", [("A", 16), ("B", 8)])
+@pytest.mark.parametrize("name,page", [("A", 16), ("B", 8), ("D", 16)])
 def test_portions_of_changing_size(dirs, plains, name, page, dtype):
     """Portions down to two tokens, cut inside pages, also without launch-by-launch graphs."""
     tokens = prompt_tokens(vocab(name), 140, 8)

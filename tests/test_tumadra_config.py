@@ -5,13 +5,13 @@ import pytest
 import torch
 
 import plain_tumadra as plain
-from tumadra_models import CONFIG_A, CONFIG_B, CONFIG_C, n_layer_runs, random_weights
+from tumadra_models import CONFIG_A, CONFIG_B, CONFIG_C, CONFIG_D, n_layer_runs, random_weights
 
 
 def test_plan_follows_the_file():
     from imparo_amd.config import plan_from_config
     from imparo_amd.engine.model import declared_tensors
-    for config in (CONFIG_A, CONFIG_B, CONFIG_C):
+    for config in (CONFIG_A, CONFIG_B, CONFIG_C, CONFIG_D):
         cfg, plan = plan_from_config(config)
         assert plan.architecture == "Tumadra" and not cfg.unread_keys
         assert [c.layer for c in plan.order] == plain.run_order(config)

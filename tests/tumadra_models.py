@@ -51,7 +51,17 @@ CONFIG_C = dict(
         layer("mamba1", dict(inner=32, state=1, dt_rank=1, conv=1), 16),
     ])
 
-CONFIGS = {"A": (CONFIG_A, 11), "B": (CONFIG_B, 12), "C": (CONFIG_C, 13)}
+# D: sizes that are no multiples of 8 (width, inner, dim, the step rank, the hidden width): under bfloat16 the
+# projections over such inner sizes run in float32
+CONFIG_D = dict(
+    architecture="Tumadra", vocab=70, width=36, norm=dict(eps=1e-5, groups=3),
+    loop=dict(start=0, stop=1, times=2),
+    layers=[
+        layer("mamba1", dict(inner=20, state=3, dt_rank=2, conv=2), 50),
+        layer("attention", attention(2, 1, 12, 20, diff=0.25, q_temp=(0.3, 16)), 28),
+    ])
+
+CONFIGS = {"A": (CONFIG_A, 11), "B": (CONFIG_B, 12), "C": (CONFIG_C, 13), "D": (CONFIG_D, 14)}
 
 
 def n_layer_runs(config):
