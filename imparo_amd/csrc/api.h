@@ -278,6 +278,8 @@ int imparo_diff_attention(const void* q, const void* k_cache, const void* v_cach
 // The same on the matrix cores, for rows that bring portions: bfloat16, pages of a multiple of 16 positions, dim
 // and vdim multiples of 4 up to 128 (imparo_diff_attention_tiles_takes). A block takes
 // imparo_diff_attention_tile() queries of one row and one head; rows of fewer than min_len tokens are skipped.
+// With dim and vdim multiples of 8 and pages of a power of two, a block stages every tile of keys and values once
+// in LDS for its four waves; otherwise every wave reads its operands itself.
 int imparo_diff_attention_tile(void);
 int imparo_diff_attention_tiles_takes(int page_size, int dim, int vdim);
 int imparo_diff_attention_tiles(const void* q, const void* k_cache, const void* v_cache, const float* gate,
