@@ -162,7 +162,7 @@ extern "C" int imparo_group_rms_norm(float* x, const float* delta, int n_delta, 
     if (!delta) n_delta = 0;
     if (n_rows == 0) return IMPARO_OK;
     const size_t delta_stride = (size_t)n_x_rows * width;
-    const int threads = WAVE * (groups < 4 ? groups : 4);
+    const int threads = WAVE * (groups < 16 ? groups : 16);      // a wave a group, up to sixteen at once
     hipStream_t s = (hipStream_t)stream;
     const int per = (width / groups + WAVE - 1) / WAVE;
     if (out_dtype == IMPARO_F32)
