@@ -1,10 +1,10 @@
-"""imparo_amd: a small, whole inference engine for one MI355X (architectures: LFM2, Tumadra)."""
-from .config import (Lfm2Config, TumadraConfig, ModelPlan, LayerPlan, LayerCall, PartSpec, register_architecture,
+"""imparo_amd: a small, whole inference engine for one MI355X (architectures: LFM2, Tumadra, Pupalorn)."""
+from .config import (Lfm2Config, TumadraConfig, PupalornConfig, ModelPlan, LayerPlan, LayerCall, PartSpec, register_architecture,
                      plan_from_config, ConfigError)
 from .parts import register_part
 from .weights import write_random_model, WeightsError
 
-__all__ = ["Lfm2Config", "TumadraConfig", "ModelPlan", "LayerPlan", "LayerCall", "PartSpec", "register_architecture",
+__all__ = ["Lfm2Config", "TumadraConfig", "PupalornConfig", "ModelPlan", "LayerPlan", "LayerCall", "PartSpec", "register_architecture",
            "plan_from_config", "ConfigError", "register_part", "write_random_model", "WeightsError",
            "Engine", "StepEntry", "generate"]
 

@@ -132,10 +132,13 @@ class PagedSpec:
         return sum(a.elements_per_position() * (4 if a.float32 else element_size) for a in self.arrays)
 
 
-def kv_spec(kv_heads: int, head_dim: int, window: Optional[int] = None, v_transposed: bool = False) -> PagedSpec:
+def kv_spec(kv_heads: int, head_dim: int, window: Optional[int] = None, v_transposed: bool = False,
+            value_dim: Optional[int] = None) -> PagedSpec:
     """Keys and values of grouped-query attention: K [kv_heads, page, head_dim]
-    and V the same, or transposed inside the page [kv_heads, head_dim, page]."""
-    v_shape = (kv_heads, head_dim, PAGE) if v_transposed else (kv_heads, PAGE, head_dim)
+    and V the same (value_dim wide where values have a size of their own), or
+    transposed inside the page [kv_heads, value_dim, page]."""
+    value_dim = head_dim if value_dim is None else value_dim
+    v_shape = (kv_heads, value_dim, PAGE) if v_transposed else (kv_heads, PAGE, value_dim)
     return PagedSpec((PagedArray("k", (kv_heads, PAGE, head_dim)), PagedArray("v", v_shape)), window)
 
 

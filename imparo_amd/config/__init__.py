@@ -10,3 +10,7 @@ from . import tumadra as _tumadra
 from .tumadra import TumadraConfig
 
 register_architecture(_tumadra.ARCHITECTURE, TumadraConfig.from_dict, _tumadra.build_plan)
+from . import pupalorn as _pupalorn
+from .pupalorn import PupalornConfig
+
+register_architecture(_pupalorn.ARCHITECTURE, PupalornConfig.from_dict, _pupalorn.build_plan)

@@ -80,6 +80,23 @@ int imparo_attention(const void* q, const void* k_cache, const void* v_cache, vo
                      int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
                      float scale, int window, int v_transposed, imparo_stream stream);
 
+// The two above for heads whose values have another size than their keys (value_dim): a token's row is
+// heads + kv_heads units of head_dim, then kv_heads units of value_dim; the value cache holds value_dim a
+// position and out is [tokens, heads * value_dim]. head_dim a multiple of 8. The store also takes rows of
+// queries only (kv_heads 0, write_kv 0), for a layer that reads another layer's keys and values.
+int imparo_qk_norm_rope_store_dv(const float* qkv, const float* q_weight, const float* k_weight, float eps,
+                                 const float* inv_freq, int n_freq, int interleaved,
+                                 const int32_t* positions, const int32_t* row_of_token,
+                                 const int32_t* block_table, int table_stride, int page_size,
+                                 void* q_out, void* k_cache, void* v_cache, int dtype, int write_kv,
+                                 int n_tokens, int heads, int kv_heads, int head_dim, int value_dim, int n_pages,
+                                 int v_transposed, imparo_stream stream);
+int imparo_attention_dv(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
+                        const int32_t* positions, const int32_t* row_of_token,
+                        const int32_t* block_table, int table_stride, int page_size,
+                        int n_tokens, int heads, int kv_heads, int head_dim, int value_dim, int n_pages,
+                        float scale, int window, int v_transposed, imparo_stream stream);
+
 // Matrix-core attention, bfloat16, V cache transposed, page_size a power of two
 // >= 16, head_dim a multiple of 16 up to 128.
 // Decode: one query token per listed row (rows[i] indexes seg_start); the key
@@ -387,6 +404,41 @@ int imparo_program_needs(ImparoProgram* p, const ImparoStepArgs* args, int64_t* 
 // imparo_program_needs says what to bind. Any other failure: imparo_program_error names the operation.
 int imparo_program_run(ImparoProgram* p, const ImparoStepArgs* args, float** logits, imparo_stream stream);
 const char* imparo_program_error(const ImparoProgram* p);
+
+// x[t] = table[ids[t]] * scale (float32 product).
+int imparo_embed_gather_scaled(const void* table, int table_dtype, const int32_t* ids, float* x,
+                               int n_tokens, int width, int vocab, float scale, imparo_stream stream);
+
+// ---- a routed feed-forward (mixture of experts)
+// route: scores = softmax(logits[t, :n_router]); the `top` largest of score + correction are chosen (of equal
+// ones the lowest index), choice [tokens, top] holds their indices and weight [tokens, top] their scores.
+int imparo_moe_route(const float* logits, const float* correction, int32_t* choice, float* weight,
+                     int n_tokens, int n_router, int top, imparo_stream stream);
+// plan: entries are (token, choice) pairs in row-major order; those whose expert is below n_experts get a slot,
+// an expert's slots side by side (slot_of_entry, -1 for the others; entry_of_slot), and `tiles` [max_tiles, 3]
+// lists (expert, first slot, rows <= tile_rows) of every tile of rows, expert -1 past the list's end.
+int imparo_moe_tile_rows(int n_entries, int n_experts, int dtype);
+int imparo_moe_max_tiles(int n_entries, int n_experts, int tile_rows);
+int imparo_moe_plan(const int32_t* choice, int n_entries, int n_experts, int tile_rows,
+                    int32_t* slot_of_entry, int32_t* entry_of_slot, int32_t* tiles, int max_tiles,
+                    imparo_stream stream);
+// product: out[slot, :n] = epilogue(a[row(slot), :k] . w[expert(slot), :n, :k]); row(slot) is the slot, or with
+// gather_div > 0 entry_of_slot[slot] / gather_div. epilogue 0: none, 1: max(z, 0)^2. bfloat16 operands (k a
+// multiple of 8, out bfloat16 or float32) or float32 throughout (tile_rows 64).
+int imparo_moe_gemm(const void* a, int a_ld, int gather_div, const int32_t* entry_of_slot, const void* w,
+                    void* out, int out_dtype, int dtype, const int32_t* tiles, int max_tiles, int tile_rows,
+                    int n, int k, int epilogue, imparo_stream stream);
+// combine: out[t] = sum_j weight[t, j] * (y[slot of (t, j)] if choice[t, j] < n_experts else h[t]), j in order.
+int imparo_moe_combine(const float* y, const void* h, int h_dtype, const int32_t* choice,
+                       const float* weight, const int32_t* slot_of_entry, float* out, int n_tokens,
+                       int width, int top, int n_experts, imparo_stream stream);
+
+// A norm on what a sublayer returns, its add into the stream, and the next norm, in one launch:
+// x[r] += rms_norm(sum of delta's slices [n_delta, n_rows_x, width])[r] * w_post; with w_next,
+// out[i] = rms_norm(x[r]) * w_next. r = rows[i] (then x is left as it is), or i.
+int imparo_post_norm_add(float* x, const float* delta, int n_delta, int n_rows_x, const int32_t* rows,
+                         const float* w_post, float eps_post, const float* w_next, float eps_next,
+                         void* out, int out_dtype, int n_out, int width, imparo_stream stream);
 
 #ifdef __cplusplus
 }

@@ -120,6 +120,7 @@ int imparo_load_code_decode_rows();
 int imparo_load_code_diff_attention();
 int imparo_load_code_elementwise();
 int imparo_load_code_gemm();
+int imparo_load_code_moe();
 int imparo_load_code_rope_cache();
 int imparo_load_code_row_ops();
 int imparo_load_code_sampling();

@@ -7,26 +7,32 @@
 // ---------------------------------------------------------------- embedding
 template <typename T>
 __global__ void k_embed_gather(const T* __restrict__ table, const int32_t* __restrict__ ids,
-                               float* __restrict__ x, int width) {
+                               float* __restrict__ x, int width, float scale) {
     const int t = blockIdx.x;
     const size_t src = (size_t)ids[t] * width;
     const size_t dst = (size_t)t * width;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) x[dst + i] = load_f32<T>(table, src + i);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) x[dst + i] = load_f32<T>(table, src + i) * scale;
 }
 
-extern "C" int imparo_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* x,
-                                   int n_tokens, int width, int vocab, imparo_stream stream) {
+// x[t] = table[ids[t]] * scale, the product in float32
+extern "C" int imparo_embed_gather_scaled(const void* table, int table_dtype, const int32_t* ids, float* x,
+                                          int n_tokens, int width, int vocab, float scale, imparo_stream stream) {
     if (!table || !ids || !x || n_tokens < 0 || width <= 0 || vocab <= 0) return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
     const int threads = width >= 1024 ? 256 : 64;
     if (table_dtype == IMPARO_F32)
-        k_embed_gather<float><<<n_tokens, threads, 0, s>>>((const float*)table, ids, x, width);
+        k_embed_gather<float><<<n_tokens, threads, 0, s>>>((const float*)table, ids, x, width, scale);
     else if (table_dtype == IMPARO_BF16)
-        k_embed_gather<bf16_t><<<n_tokens, threads, 0, s>>>((const bf16_t*)table, ids, x, width);
+        k_embed_gather<bf16_t><<<n_tokens, threads, 0, s>>>((const bf16_t*)table, ids, x, width, scale);
     else
         return IMPARO_BAD_ARGUMENT;
     return launch_status();
+}
+
+extern "C" int imparo_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* x,
+                                   int n_tokens, int width, int vocab, imparo_stream stream) {
+    return imparo_embed_gather_scaled(table, table_dtype, ids, x, n_tokens, width, vocab, 1.0f, stream);
 }
 
 // Token ids that are still on the device (sampled by the step before, not yet read back):

@@ -1,0 +1,500 @@
+// A routed feed-forward (mixture of experts) in five launches:
+//   route    softmax over the router's outputs, the choice of `top` of them by score + correction,
+//            the weights (the scores themselves, as they are), one wave a token;
+//   plan     one block: how many (token, choice) entries each expert got, a slot for every entry
+//            (the entries of one expert side by side), and the list of row tiles the products walk;
+//   product  twice: a tile of one expert's slots times that expert's matrix (up with the activation
+//            in its epilogue, then down), on the matrix cores in bfloat16, plain fused multiply-adds
+//            in float32; the grid is sized by a bound that the host knows (no count comes back);
+//   combine  a token's result: its chosen experts' rows times their weights, added in the order of
+//            the choice; an expert past the last real one passes the token's input through.
+// Which slot an entry gets depends on the order in which threads arrive; no result does: a row of
+// a product is summed over k in one order wherever the row lies in its tile, and a token's sum
+// over its experts runs in the order of its own choice.
+#include "common.h"
+#include "api.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define MOE_MAX_ROUTER 512          // router outputs (experts of both kinds)
+#define MOE_MAX_EXPERTS 1024        // real experts the plan kernel keeps counters for
+#define MOE_MAX_TOP 16
+
+// ---------------------------------------------------------------- route
+__global__ void k_moe_route(const float* __restrict__ logits, const float* __restrict__ correction,
+                            int32_t* __restrict__ choice, float* __restrict__ weight, int n_tokens, int n_router,
+                            int top) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (t >= n_tokens) return;
+    constexpr int PER = MOE_MAX_ROUTER / WAVE;
+    float z[PER], pick[PER];
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = lane + j * WAVE;
+        z[j] = i < n_router ? logits[(size_t)t * n_router + i] : -INFINITY;
+        m = fmaxf(m, z[j]);
+    }
+    m = wave_max(m);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        z[j] = (lane + j * WAVE) < n_router ? expf(z[j] - m) : 0.f;
+        sum += z[j];
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = lane + j * WAVE;
+        z[j] *= inv;
+        pick[j] = i < n_router ? z[j] + (correction ? correction[i] : 0.f) : -INFINITY;
+    }
+    for (int k = 0; k < top; ++k) {
+        // the largest choice score that is left; of equal ones the lowest index
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int i = lane + j * WAVE;
+            if (pick[j] > best) { best = pick[j]; at = i; }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, WAVE);
+            const int oa = __shfl_xor(at, off, WAVE);
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+        }
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < PER; ++j)
+            if (lane + j * WAVE == at) { s = z[j]; pick[j] = -INFINITY; }
+        s = wave_sum(s);           // one lane holds it
+        if (lane == 0) {
+            choice[(size_t)t * top + k] = at;
+            weight[(size_t)t * top + k] = s;
+        }
+    }
+}
+
+extern "C" int imparo_moe_route(const float* logits, const float* correction, int32_t* choice, float* weight,
+                                int n_tokens, int n_router, int top, imparo_stream stream) {
+    if (!logits || !choice || !weight || n_tokens < 0) return IMPARO_BAD_ARGUMENT;
+    if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > n_router || top > MOE_MAX_TOP)
+        return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    k_moe_route<<<(n_tokens + 3) / 4, 4 * WAVE, 0, (hipStream_t)stream>>>(logits, correction, choice, weight, n_tokens,
+                                                                         n_router, top);
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- plan
+// tiles[3 i ..]: expert, first slot, rows of tile i; expert -1 where the list has ended.
+__global__ __launch_bounds__(1024) void k_moe_plan(const int32_t* __restrict__ choice, int n_entries, int n_experts,
+                                                   int tile_rows, int32_t* __restrict__ slot_of_entry,
+                                                   int32_t* __restrict__ entry_of_slot, int32_t* __restrict__ tiles,
+                                                   int max_tiles) {
+    __shared__ int count[MOE_MAX_EXPERTS], first[MOE_MAX_EXPERTS], first_tile[MOE_MAX_EXPERTS + 1];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < n_experts; e += blockDim.x) count[e] = 0;
+    __syncthreads();
+    for (int i = tid; i < n_entries; i += blockDim.x) {
+        const int e = choice[i];
+        if (e >= 0 && e < n_experts) atomicAdd(&count[e], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int slots = 0, n_tiles = 0;
+        for (int e = 0; e < n_experts; ++e) {
+            first[e] = slots;
+            first_tile[e] = n_tiles;
+            slots += count[e];
+            n_tiles += (count[e] + tile_rows - 1) / tile_rows;
+        }
+        first_tile[n_experts] = n_tiles;
+    }
+    __syncthreads();
+    for (int e = tid; e < n_experts; e += blockDim.x) {
+        const int n = count[e];
+        int i = first_tile[e];
+        for (int r = 0; r < n && i < max_tiles; r += tile_rows, ++i) {
+            tiles[3 * i] = e;
+            tiles[3 * i + 1] = first[e] + r;
+            tiles[3 * i + 2] = min(tile_rows, n - r);
+        }
+    }
+    for (int i = first_tile[n_experts] + tid; i < max_tiles; i += blockDim.x) {
+        tiles[3 * i] = -1;
+        tiles[3 * i + 1] = 0;
+        tiles[3 * i + 2] = 0;
+    }
+    __syncthreads();
+    for (int e = tid; e < n_experts; e += blockDim.x) count[e] = 0;      // now the cursor of each expert
+    __syncthreads();
+    for (int i = tid; i < n_entries; i += blockDim.x) {
+        const int e = choice[i];
+        int slot = -1;
+        if (e >= 0 && e < n_experts) {
+            slot = first[e] + atomicAdd(&count[e], 1);
+            entry_of_slot[slot] = i;
+        }
+        slot_of_entry[i] = slot;
+    }
+}
+
+extern "C" int imparo_moe_max_tiles(int n_entries, int n_experts, int tile_rows) {
+    if (n_entries <= 0 || tile_rows <= 0) return 0;
+    return (n_entries + tile_rows - 1) / tile_rows + (n_experts < n_entries ? n_experts : n_entries);
+}
+
+// Rows of a product's tile for this many entries over this many experts: the wide tile where an
+// expert's share fills it, the narrow one else (a decode step, many experts).
+extern "C" int imparo_moe_tile_rows(int n_entries, int n_experts, int dtype) {
+    if (dtype != IMPARO_BF16) return 64;
+    return (n_experts > 0 && n_entries / n_experts >= 96) ? 128 : 64;
+}
+
+extern "C" int imparo_moe_plan(const int32_t* choice, int n_entries, int n_experts, int tile_rows,
+                               int32_t* slot_of_entry, int32_t* entry_of_slot, int32_t* tiles, int max_tiles,
+                               imparo_stream stream) {
+    if (!choice || !slot_of_entry || !entry_of_slot || !tiles || n_entries < 0) return IMPARO_BAD_ARGUMENT;
+    if (n_experts < 0 || n_experts > MOE_MAX_EXPERTS || tile_rows < 1) return IMPARO_BAD_ARGUMENT;
+    if (max_tiles < imparo_moe_max_tiles(n_entries, n_experts, tile_rows)) return IMPARO_SCRATCH_TOO_SMALL;
+    if (n_entries == 0) return IMPARO_OK;
+    k_moe_plan<<<1, 1024, 0, (hipStream_t)stream>>>(choice, n_entries, n_experts, tile_rows, slot_of_entry,
+                                                    entry_of_slot, tiles, max_tiles);
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- products
+#define MOE_EPI_NONE 0
+#define MOE_EPI_RELU2 1        // max(z, 0)^2
+
+__device__ __forceinline__ float moe_epilogue(float v, int epi) {
+    if (epi == MOE_EPI_RELU2) {
+        v = fmaxf(v, 0.f);
+        v *= v;
+    }
+    return v;
+}
+
+union MoeFrag {
+    uint4 u;
+    bf16x8 v;
+};
+
+// out[slot, n] = epi(sum_k a[row(slot), k] * w[expert, n, k]) for the slots of one tile. row(slot) is the
+// slot itself, or with gather_div the token of the slot's entry (entry / gather_div). Four waves as 2 x 2,
+// each WM x WN products of 32 x 32; K in steps of 64 through two LDS stages, the next step's loads in
+// registers while this one is multiplied. K is a multiple of 8.
+template <int WM, int WN, typename TOut>
+__global__ __launch_bounds__(256) void k_moe_gemm_bf16(const bf16_t* __restrict__ A, int a_ld, int gather_div,
+                                                       const int32_t* __restrict__ entry_of_slot,
+                                                       const bf16_t* __restrict__ W, TOut* __restrict__ out,
+                                                       const int32_t* __restrict__ tiles, int N, int K, int epi) {
+    constexpr int TM = 64 * WM, TN = 64 * WN, LD = 72, BK = 64;
+    __shared__ __attribute__((aligned(16))) bf16_t As[2][TM * LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Bs[2][TN * LD];
+    const int expert = tiles[3 * blockIdx.x];
+    if (expert < 0) return;
+    const int row0 = tiles[3 * blockIdx.x + 1], rows = tiles[3 * blockIdx.x + 2];
+    const int n0 = blockIdx.y * TN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const bf16_t* Wb = W + (size_t)expert * N * K;
+    const int kc = (tid & 7) * 8;
+    const bf16_t* pa[TM / 32];
+    const bf16_t* pb[TN / 32];
+#pragma unroll
+    for (int j = 0; j < TM / 32; ++j) {
+        const int slot = row0 + min((tid >> 3) + 32 * j, rows - 1);
+        const int src = gather_div ? entry_of_slot[slot] / gather_div : slot;
+        pa[j] = A + (size_t)src * a_ld;
+    }
+#pragma unroll
+    for (int j = 0; j < TN / 32; ++j) pb[j] = Wb + (size_t)min(n0 + (tid >> 3) + 32 * j, N - 1) * K;
+    uint4 ra[TM / 32], rb[TN / 32];
+    const uint4 zero = {0u, 0u, 0u, 0u};
+    auto fetch = [&](int kt) {
+        const int k = kt * BK + kc;
+        const bool in = k < K;
+        const int kk = in ? k : 0;
+#pragma unroll
+        for (int j = 0; j < TM / 32; ++j) {
+            const uint4 v = *reinterpret_cast<const uint4*>(pa[j] + kk);
+            ra[j] = in ? v : zero;
+        }
+#pragma unroll
+        for (int j = 0; j < TN / 32; ++j) {
+            const uint4 v = *reinterpret_cast<const uint4*>(pb[j] + kk);
+            rb[j] = in ? v : zero;
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < TM / 32; ++j)
+            *reinterpret_cast<uint4*>(&As[buf][((tid >> 3) + 32 * j) * LD + kc]) = ra[j];
+#pragma unroll
+        for (int j = 0; j < TN / 32; ++j)
+            *reinterpret_cast<uint4*>(&Bs[buf][((tid >> 3) + 32 * j) * LD + kc]) = rb[j];
+    };
+    f32x16 acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    const int a_base = (wm * 32 * WM + (lane & 31)) * LD + (lane >> 5) * 8;
+    const int b_base = (wn * 32 * WN + (lane & 31)) * LD + (lane >> 5) * 8;
+    const int nk = (K + BK - 1) / BK;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) fetch(kt + 1);
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            MoeFrag fa[WM], fb[WN];
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+                fa[i].u = *reinterpret_cast<const uint4*>(&As[buf][a_base + i * 32 * LD + ks * 16]);
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+                fb[j].u = *reinterpret_cast<const uint4*>(&Bs[buf][b_base + j * 32 * LD + ks * 16]);
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int j = 0; j < WN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i].v, fb[j].v, acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) stash(buf ^ 1);
+        __syncthreads();
+    }
+    // a lane holds column lane % 32 of a 32 x 32 product, rows 8 (r / 4) + 4 (lane / 32) + r % 4
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+            const int n = n0 + wn * 32 * WN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = wm * 32 * WM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < rows && n < N) store_f32<TOut>(out, (size_t)(row0 + m) * N + n, moe_epilogue(acc[i][j][r], epi));
+            }
+        }
+}
+
+// The same in float32: a tile of 64 slots by 64 outputs, K in steps of 16 through LDS, every output
+// summed over k = 0, 1, 2, ... by fused multiply-adds, whatever the tile holds beside it.
+__global__ __launch_bounds__(256) void k_moe_gemm_f32(const float* __restrict__ A, int a_ld, int gather_div,
+                                                      const int32_t* __restrict__ entry_of_slot,
+                                                      const float* __restrict__ W, float* __restrict__ out,
+                                                      const int32_t* __restrict__ tiles, int N, int K, int epi) {
+    constexpr int TM = 64, TN = 64, BK = 16, LD = 68;
+    __shared__ float As[BK][LD], Bs[BK][LD];
+    const int expert = tiles[3 * blockIdx.x];
+    if (expert < 0) return;
+    const int row0 = tiles[3 * blockIdx.x + 1], rows = tiles[3 * blockIdx.x + 2];
+    const int n0 = blockIdx.y * TN;
+    const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
+    const float* Wb = W + (size_t)expert * N * K;
+    const float* pa[4];
+    const float* pb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int r = (tid >> 4) + 16 * j;
+        const int slot = row0 + min(r, rows - 1);
+        const int src = gather_div ? entry_of_slot[slot] / gather_div : slot;
+        pa[j] = A + (size_t)src * a_ld;
+        pb[j] = Wb + (size_t)min(n0 + r, N - 1) * K;
+    }
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        const int k = k0 + tx;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            As[tx][(tid >> 4) + 16 * j] = k < K ? pa[j][k] : 0.f;
+            Bs[tx][(tid >> 4) + 16 * j] = k < K ? pb[j][k] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BK; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int m = ty * 4 + i, n = n0 + tx * 4 + j;
+            if (m < rows && n < N) out[(size_t)(row0 + m) * N + n] = moe_epilogue(acc[i][j], epi);
+        }
+}
+
+extern "C" int imparo_moe_gemm(const void* a, int a_ld, int gather_div, const int32_t* entry_of_slot, const void* w,
+                               void* out, int out_dtype, int dtype, const int32_t* tiles, int max_tiles, int tile_rows,
+                               int n, int k, int epilogue, imparo_stream stream) {
+    if (!a || !w || !out || !tiles || max_tiles < 0 || n < 1 || k < 1 || a_ld < k || gather_div < 0)
+        return IMPARO_BAD_ARGUMENT;
+    if (gather_div && !entry_of_slot) return IMPARO_BAD_ARGUMENT;
+    if (epilogue != MOE_EPI_NONE && epilogue != MOE_EPI_RELU2) return IMPARO_BAD_ARGUMENT;
+    if (max_tiles == 0) return IMPARO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == IMPARO_F32) {
+        if (out_dtype != IMPARO_F32 || tile_rows != 64) return IMPARO_BAD_ARGUMENT;
+        k_moe_gemm_f32<<<dim3(max_tiles, (n + 63) / 64), 256, 0, s>>>((const float*)a, a_ld, gather_div, entry_of_slot,
+                                                                     (const float*)w, (float*)out, tiles, n, k, epilogue);
+        return launch_status();
+    }
+    if (dtype != IMPARO_BF16 || k % 8 || a_ld % 8 || ((uintptr_t)a | (uintptr_t)w) % 16) return IMPARO_BAD_ARGUMENT;
+#define MOE_LAUNCH(WM, WN, TO)                                                                                       \
+    k_moe_gemm_bf16<WM, WN, TO><<<dim3(max_tiles, (n + 64 * WN - 1) / (64 * WN)), 256, 0, s>>>(                      \
+        (const bf16_t*)a, a_ld, gather_div, entry_of_slot, (const bf16_t*)w, (TO*)out, tiles, n, k, epilogue)
+    if (tile_rows == 128) {
+        if (out_dtype == IMPARO_BF16) MOE_LAUNCH(2, 2, bf16_t);
+        else if (out_dtype == IMPARO_F32) MOE_LAUNCH(2, 2, float);
+        else return IMPARO_BAD_ARGUMENT;
+    } else if (tile_rows == 64) {
+        if (n >= 128) {
+            if (out_dtype == IMPARO_BF16) MOE_LAUNCH(1, 2, bf16_t);
+            else if (out_dtype == IMPARO_F32) MOE_LAUNCH(1, 2, float);
+            else return IMPARO_BAD_ARGUMENT;
+        } else {
+            if (out_dtype == IMPARO_BF16) MOE_LAUNCH(1, 1, bf16_t);
+            else if (out_dtype == IMPARO_F32) MOE_LAUNCH(1, 1, float);
+            else return IMPARO_BAD_ARGUMENT;
+        }
+    } else {
+        return IMPARO_BAD_ARGUMENT;
+    }
+#undef MOE_LAUNCH
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- combine
+// out[t] = sum over the token's choices, in their order, of weight * (the expert's row, or for an
+// expert past the last real one the token's input).
+template <typename T>
+__global__ void k_moe_combine(const float* __restrict__ y, const T* __restrict__ h, const int32_t* __restrict__ choice,
+                              const float* __restrict__ weight, const int32_t* __restrict__ slot_of_entry,
+                              float* __restrict__ out, int width, int top, int n_experts) {
+    const int t = blockIdx.x;
+    __shared__ int slot[MOE_MAX_TOP];
+    __shared__ float w[MOE_MAX_TOP];
+    if (threadIdx.x < top) {
+        const int e = choice[(size_t)t * top + threadIdx.x];
+        slot[threadIdx.x] = e < n_experts ? slot_of_entry[(size_t)t * top + threadIdx.x] : -1;
+        w[threadIdx.x] = weight[(size_t)t * top + threadIdx.x];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float acc = 0.f;
+        for (int k = 0; k < top; ++k) {
+            const float v = slot[k] >= 0 ? y[(size_t)slot[k] * width + i] : load_f32<T>(h, (size_t)t * width + i);
+            acc = fmaf(w[k], v, acc);
+        }
+        out[(size_t)t * width + i] = acc;
+    }
+}
+
+extern "C" int imparo_moe_combine(const float* y, const void* h, int h_dtype, const int32_t* choice,
+                                  const float* weight, const int32_t* slot_of_entry, float* out, int n_tokens,
+                                  int width, int top, int n_experts, imparo_stream stream) {
+    if (!y || !h || !choice || !weight || !slot_of_entry || !out || n_tokens < 0 || width < 1) return IMPARO_BAD_ARGUMENT;
+    if (top < 1 || top > MOE_MAX_TOP || n_experts < 0) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = width >= 1024 ? 256 : 64;
+    if (h_dtype == IMPARO_F32)
+        k_moe_combine<float><<<n_tokens, threads, 0, s>>>(y, (const float*)h, choice, weight, slot_of_entry, out, width,
+                                                          top, n_experts);
+    else if (h_dtype == IMPARO_BF16)
+        k_moe_combine<bf16_t><<<n_tokens, threads, 0, s>>>(y, (const bf16_t*)h, choice, weight, slot_of_entry, out,
+                                                           width, top, n_experts);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- a norm on what a sublayer returns
+// x[row] += d / sqrt(mean(d^2) + eps_post) * w_post, d = the sum of the delta's slices in order; then,
+// with w_next, out[row] = x[row] / sqrt(mean(x[row]^2) + eps_next) * w_next. One block a row, the row in
+// LDS between the passes, every sum in float32 and in an order that the width alone decides. With `rows`
+// only those rows are taken and the stream is left as it is (the rows whose logits are wanted).
+template <typename TOut>
+__global__ __launch_bounds__(256) void k_post_norm_add(float* __restrict__ x, const float* __restrict__ delta,
+                                                       int n_delta, size_t delta_stride,
+                                                       const int32_t* __restrict__ rows,
+                                                       const float* __restrict__ w_post, float eps_post,
+                                                       const float* __restrict__ w_next, float eps_next,
+                                                       TOut* __restrict__ out, int width, int write_back) {
+    extern __shared__ float row[];
+    __shared__ float scratch[16];
+    const int i_out = blockIdx.x;
+    const size_t src = (size_t)(rows ? rows[i_out] : i_out) * width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float d = delta[src + i];
+        for (int s = 1; s < n_delta; ++s) d += delta[(size_t)s * delta_stride + src + i];
+        row[i] = d;
+        ss = fmaf(d, d, ss);
+    }
+    const float r1 = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps_post);
+    ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float v = x[src + i] + row[i] * r1 * w_post[i];
+        row[i] = v;
+        if (write_back) x[src + i] = v;
+        ss = fmaf(v, v, ss);
+    }
+    if (!w_next) return;
+    const float r2 = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps_next);
+    for (int i = threadIdx.x; i < width; i += blockDim.x)
+        store_f32<TOut>(out, (size_t)i_out * width + i, row[i] * r2 * w_next[i]);
+}
+
+extern "C" int imparo_post_norm_add(float* x, const float* delta, int n_delta, int n_rows_x, const int32_t* rows,
+                                    const float* w_post, float eps_post, const float* w_next, float eps_next,
+                                    void* out, int out_dtype, int n_out, int width, imparo_stream stream) {
+    if (!x || !delta || !w_post || n_delta < 1 || n_rows_x < 0 || n_out < 0 || width < 1 || width > 16384)
+        return IMPARO_BAD_ARGUMENT;
+    if (w_next && !out) return IMPARO_BAD_ARGUMENT;
+    if (!rows && n_out != n_rows_x) return IMPARO_BAD_ARGUMENT;
+    if (n_out == 0) return IMPARO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const size_t stride = (size_t)n_rows_x * width;
+    const int write_back = rows ? 0 : 1;
+    const size_t lds = (size_t)width * sizeof(float);
+    if (!w_next || out_dtype == IMPARO_F32)
+        k_post_norm_add<float><<<n_out, 256, lds, s>>>(x, delta, n_delta, stride, rows, w_post, eps_post, w_next,
+                                                       eps_next, (float*)out, width, write_back);
+    else if (out_dtype == IMPARO_BF16)
+        k_post_norm_add<bf16_t><<<n_out, 256, lds, s>>>(x, delta, n_delta, stride, rows, w_post, eps_post, w_next,
+                                                        eps_next, (bf16_t*)out, width, write_back);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
+int imparo_load_code_moe() {
+    hipFuncAttributes attributes;
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_moe_plan)) == hipSuccess ? IMPARO_OK
+                                                                                                       : IMPARO_LAUNCH_FAILED;
+}

@@ -36,8 +36,8 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
                                      const int32_t* __restrict__ positions, const int32_t* __restrict__ row_of_token,
                                      const int32_t* __restrict__ block_table, int table_stride, int page_size,
                                      T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                     int write_kv, int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
-                                     int v_transposed) {
+                                     int write_kv, int n_tokens, int heads, int kv_heads, int head_dim, int value_dim,
+                                     int n_pages, int v_transposed) {
     __shared__ float rows[ROPE_WAVES][ROPE_MAX_HEAD_DIM];
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = threadIdx.x / WAVE;
@@ -46,10 +46,15 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
     if (id >= (long long)n_tokens * units) return;
     const int t = (int)(id / units);
     const int u = (int)(id - (long long)t * units);
-    const float* src = qkv + (size_t)t * units * head_dim + (size_t)u * head_dim;
     float* row = rows[wave];
     const bool is_q = u < heads;
     const bool is_v = u >= heads + kv_heads;
+    // a token's row: heads + kv_heads units of head_dim, then kv_heads units of value_dim
+    const size_t row_width = (size_t)(heads + kv_heads) * head_dim + (size_t)kv_heads * value_dim;
+    const float* src = qkv + (size_t)t * row_width +
+                       (is_v ? (size_t)(heads + kv_heads) * head_dim + (size_t)(u - heads - kv_heads) * value_dim
+                             : (size_t)u * head_dim);
+    const int unit_dim = is_v ? value_dim : head_dim;
     const float* weight = is_q ? q_weight : k_weight;
 
     // Everything the wave needs is asked for before the first value is used: what a decode
@@ -63,7 +68,7 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
 #pragma unroll
     for (int j = 0; j < PER_LANE; ++j) {
         const int i = lane + j * WAVE;
-        a[j] = i < head_dim ? src[i] : 0.f;
+        a[j] = i < unit_dim ? src[i] : 0.f;
         w[j] = (i < head_dim && weight && !is_v) ? weight[i] : 1.f;
         freq[j] = (i < n_freq && !is_v) ? inv_freq[i] : 0.f;
     }
@@ -98,7 +103,7 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
 #pragma unroll
         for (int j = 0; j < PER_LANE; ++j) {
             const int i = lane + j * WAVE;
-            if (i < head_dim) row[i] = a[j];
+            if (i < value_dim) row[i] = a[j];
         }
     }
     wave_lds_sync();
@@ -113,13 +118,13 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
     if (page < 0 || page >= n_pages) return;   // never write outside the pool
     if (is_v && v_transposed) {
         // [page, kv head, dim, slot]: the keys of one dimension lie side by side
-        T* dst = v_cache + ((size_t)page * kv_heads + kvh) * page_size * head_dim + (pos % page_size);
-        for (int i = lane; i < head_dim; i += WAVE) store_f32<T>(dst, (size_t)i * page_size, row[i]);
+        T* dst = v_cache + ((size_t)page * kv_heads + kvh) * page_size * value_dim + (pos % page_size);
+        for (int i = lane; i < value_dim; i += WAVE) store_f32<T>(dst, (size_t)i * page_size, row[i]);
         return;
     }
     T* cache = is_v ? v_cache : k_cache;
-    T* dst = cache + (((size_t)page * kv_heads + kvh) * page_size + (pos % page_size)) * head_dim;
-    for (int i = lane; i < head_dim; i += WAVE) store_f32<T>(dst, i, row[i]);
+    T* dst = cache + (((size_t)page * kv_heads + kvh) * page_size + (pos % page_size)) * unit_dim;
+    for (int i = lane; i < unit_dim; i += WAVE) store_f32<T>(dst, i, row[i]);
 }
 
 // The same for many tokens (a prompt's portion): one block per token. The rotation's sines and
@@ -368,17 +373,21 @@ static void launch_rope_token(const float* qkv, const float* q_weight, const flo
 #define ROPE_TOKEN_KERNEL_FROM 96
 #endif
 
-extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight, const float* k_weight, float eps,
+// The row of a token holds heads + kv_heads units of head_dim (queries, keys) and kv_heads units of
+// value_dim (values); kv_heads 0 (with write_kv 0): a row of queries only, for a layer that reads
+// another layer's keys and values.
+extern "C" int imparo_qk_norm_rope_store_dv(const float* qkv, const float* q_weight, const float* k_weight, float eps,
                                          const float* inv_freq, int n_freq, int interleaved,
                                          const int32_t* positions, const int32_t* row_of_token,
                                          const int32_t* block_table, int table_stride, int page_size,
                                          void* q_out, void* k_cache, void* v_cache, int dtype, int write_kv,
-                                         int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
-                                         int v_transposed, imparo_stream stream) {
+                                         int n_tokens, int heads, int kv_heads, int head_dim, int value_dim,
+                                         int n_pages, int v_transposed, imparo_stream stream) {
     if (!qkv || !positions || !q_out) return IMPARO_BAD_ARGUMENT;
     if (write_kv && (!row_of_token || !block_table || !k_cache || !v_cache)) return IMPARO_BAD_ARGUMENT;
-    if (n_tokens < 0 || heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim > ROPE_MAX_HEAD_DIM)
+    if (n_tokens < 0 || heads <= 0 || kv_heads < 0 || head_dim <= 0 || head_dim > ROPE_MAX_HEAD_DIM)
         return IMPARO_BAD_ARGUMENT;
+    if ((write_kv && kv_heads == 0) || value_dim <= 0 || value_dim > ROPE_MAX_HEAD_DIM) return IMPARO_BAD_ARGUMENT;
     if (n_freq < 0 || 2 * n_freq > head_dim || (n_freq > 0 && !inv_freq)) return IMPARO_BAD_ARGUMENT;
     if (page_size <= 0 || table_stride < 0 || n_pages < 0) return IMPARO_BAD_ARGUMENT;
     if ((q_weight == nullptr) != (k_weight == nullptr)) return IMPARO_BAD_ARGUMENT;
@@ -386,7 +395,7 @@ extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight
     const long long total = (long long)n_tokens * (heads + 2 * kv_heads);
     const unsigned blocks = (unsigned)((total + ROPE_WAVES - 1) / ROPE_WAVES);
     hipStream_t s = (hipStream_t)stream;
-    if (n_tokens >= ROPE_TOKEN_KERNEL_FROM && (dtype == IMPARO_F32 || dtype == IMPARO_BF16)) {
+    if (n_tokens >= ROPE_TOKEN_KERNEL_FROM && value_dim == head_dim && (dtype == IMPARO_F32 || dtype == IMPARO_BF16)) {
         if (dtype == IMPARO_F32)
             launch_rope_token<float>(qkv, q_weight, k_weight, eps, inv_freq, n_freq, interleaved, positions, row_of_token,
                                      block_table, table_stride, page_size, (float*)q_out, (float*)k_cache,
@@ -403,15 +412,29 @@ extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight
         k_qk_norm_rope_store<float><<<blocks, ROPE_WAVES * WAVE, 0, s>>>(
             qkv, q_weight, k_weight, eps, inv_freq, n_freq, interleaved, positions, row_of_token, block_table, table_stride,
             page_size, (float*)q_out, (float*)k_cache, (float*)v_cache, write_kv, n_tokens, heads, kv_heads,
-            head_dim, n_pages, v_transposed);
+            head_dim, value_dim, n_pages, v_transposed);
     else if (dtype == IMPARO_BF16)
         k_qk_norm_rope_store<bf16_t><<<blocks, ROPE_WAVES * WAVE, 0, s>>>(
             qkv, q_weight, k_weight, eps, inv_freq, n_freq, interleaved, positions, row_of_token, block_table, table_stride,
             page_size, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, write_kv, n_tokens, heads, kv_heads,
-            head_dim, n_pages, v_transposed);
+            head_dim, value_dim, n_pages, v_transposed);
     else
         return IMPARO_BAD_ARGUMENT;
     return launch_status();
+}
+
+extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight, const float* k_weight, float eps,
+                                         const float* inv_freq, int n_freq, int interleaved,
+                                         const int32_t* positions, const int32_t* row_of_token,
+                                         const int32_t* block_table, int table_stride, int page_size,
+                                         void* q_out, void* k_cache, void* v_cache, int dtype, int write_kv,
+                                         int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
+                                         int v_transposed, imparo_stream stream) {
+    if (kv_heads <= 0) return IMPARO_BAD_ARGUMENT;
+    return imparo_qk_norm_rope_store_dv(qkv, q_weight, k_weight, eps, inv_freq, n_freq, interleaved, positions,
+                                        row_of_token, block_table, table_stride, page_size, q_out, k_cache, v_cache,
+                                        dtype, write_kv, n_tokens, heads, kv_heads, head_dim, head_dim, n_pages,
+                                        v_transposed, stream);
 }
 
 // Asks the runtime about one kernel of this file, which makes it load the file's code onto the

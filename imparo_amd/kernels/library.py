@@ -65,6 +65,18 @@ _SIGNATURES = {
     "imparo_diff_attention_tile": [],
     "imparo_diff_attention_tiles_takes": [I, I, I],
     "imparo_diff_attention_tiles": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, I, F, F, F, I, P],
+    "imparo_embed_gather_scaled": [P, I, P, P, I, I, I, F, P],
+    "imparo_qk_norm_rope_store_dv": [P, P, P, F, P, I, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, P],
+    "imparo_attention_dv": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, P],
+    "imparo_moe_route": [P, P, P, P, I, I, I, P],
+    "imparo_moe_tile_rows": [I, I, I],
+    "imparo_moe_max_tiles": [I, I, I],
+    "imparo_moe_plan": [P, I, I, I, P, P, P, I, P],
+    # a, a_ld, gather_div, entry_of_slot, w, out, out_dtype, dtype, tiles, max_tiles, tile_rows, n, k, epilogue, stream
+    "imparo_moe_gemm": [P, I, I, P, P, P, I, I, P, I, I, I, I, I, P],
+    "imparo_moe_combine": [P, P, I, P, P, P, P, I, I, I, I, P],
+    # x, delta, n_delta, n_rows_x, rows, w_post, eps_post, w_next, eps_next, out, out_dtype, n_out, width, stream
+    "imparo_post_norm_add": [P, P, I, I, P, P, F, P, F, P, I, I, I, P],
     "imparo_rows_parts": [I],
     # x, ssq_in, n_parts, eps, w, bias, y, out_dtype, x_io, ssq_out, weighted_out, weighted_by, m, n, k, epilogue, stream
     "imparo_rows_gemm": [P, P, I, F, P, P, P, I, P, P, P, P, I, I, I, I, P],

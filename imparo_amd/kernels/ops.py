@@ -84,13 +84,14 @@ def load_code() -> None:
     _check(library().imparo_load_code(), "load_code")
 
 
-def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale in float32."""
     vocab, width = table.shape
     n = ids.shape[0]
-    _check(library().imparo_embed_gather(
+    _check(library().imparo_embed_gather_scaled(
         _dev(table, "embedding table"), _code(table, "embedding table"),
         _dev(ids, "token ids", torch.int32, (n,)), _dev(out, "embedding output", torch.float32, (n, width)),
-        n, width, vocab, _stream()), "embed_gather")
+        n, width, vocab, float(scale), _stream()), "embed_gather")
     return out
 
 
@@ -185,11 +186,13 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_we
                        row_of_token: torch.Tensor, block_table: Optional[torch.Tensor], page_size: int,
                        q_out: torch.Tensor, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                        heads: int, kv_heads: int, head_dim: int, v_transposed: bool = False,
-                       interleaved: bool = False) -> torch.Tensor:
+                       interleaved: bool = False, value_dim: Optional[int] = None) -> torch.Tensor:
     """`inv_freq` [n] turns pair i by position * inv_freq[i]: pair i is dims (i, i + n), or with
-    `interleaved` dims (2i, 2i + 1)."""
+    `interleaved` dims (2i, 2i + 1). `value_dim`: the size of a head's values where it is not
+    head_dim (the row then ends in kv_heads units of that size). kv_heads 0: rows of queries only."""
     n = qkv.shape[0]
-    units = heads + 2 * kv_heads
+    value_dim = head_dim if value_dim is None else int(value_dim)
+    row_width = (heads + kv_heads) * head_dim + kv_heads * value_dim
     write_kv = k_cache is not None
     n_freq = 0 if inv_freq is None else inv_freq.shape[0]
     n_pages = 0
@@ -197,21 +200,21 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_we
     if write_kv:
         n_pages = k_cache.shape[0]
         _dev(k_cache, "k cache", q_out.dtype, (n_pages, kv_heads, page_size, head_dim))
-        _dev(v_cache, "v cache", q_out.dtype, (n_pages, kv_heads, head_dim, page_size) if v_transposed
-             else (n_pages, kv_heads, page_size, head_dim))
+        _dev(v_cache, "v cache", q_out.dtype, (n_pages, kv_heads, value_dim, page_size) if v_transposed
+             else (n_pages, kv_heads, page_size, value_dim))
         if block_table is None or block_table.dim() != 2:
             raise KernelArgumentError("qk_norm_rope_store: a [rows, pages] block table is needed to write the cache")
         table_stride = block_table.shape[1]
-    _check(library().imparo_qk_norm_rope_store(
-        _dev(qkv, "qkv", torch.float32, (n, units * head_dim)),
+    _check(library().imparo_qk_norm_rope_store_dv(
+        _dev(qkv, "qkv", torch.float32, (n, row_width)),
         _dev(q_weight, "q norm weight", torch.float32, (head_dim,)),
         _dev(k_weight, "k norm weight", torch.float32, (head_dim,)), float(eps),
         _dev(inv_freq, "inverse frequencies", torch.float32), n_freq, int(interleaved),
         _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
         _dev(block_table, "block table", torch.int32), table_stride, page_size,
         _dev(q_out, "q out", None, (n, heads, head_dim)), _dev(k_cache, "k cache"), _dev(v_cache, "v cache"),
-        _code(q_out, "q out"), int(write_kv), n, heads, kv_heads, head_dim, n_pages, int(v_transposed), _stream()),
-        "qk_norm_rope_store")
+        _code(q_out, "q out"), int(write_kv), n, heads, kv_heads, head_dim, value_dim, n_pages, int(v_transposed),
+        _stream()), "qk_norm_rope_store")
     return q_out
 
 
@@ -222,20 +225,22 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out
     float32 or bfloat16; one wave per (token, head)."""
     n, heads, head_dim = q.shape
     n_pages, kv_heads, page_size, hd = k_cache.shape
+    value_dim = v_cache.shape[2] if v_transposed else v_cache.shape[3]
     if hd != head_dim:
         raise KernelArgumentError(f"attention: q has head size {head_dim}, the cache {hd}")
-    if head_dim % 16 != 0:
-        raise KernelArgumentError(f"attention: head size must be a multiple of 16, got {head_dim}")
+    if head_dim % 8 != 0:
+        raise KernelArgumentError(f"attention: head size must be a multiple of 8, got {head_dim}")
     if heads % kv_heads != 0:
         raise KernelArgumentError(f"attention: {heads} heads cannot share {kv_heads} kv heads evenly")
-    _check(library().imparo_attention(
+    _check(library().imparo_attention_dv(
         _dev(q, "q"), _dev(k_cache, "k cache", q.dtype),
-        _dev(v_cache, "v cache", q.dtype, (n_pages, kv_heads, head_dim, page_size) if v_transposed else k_cache.shape),
-        _dev(out, "attention out", q.dtype, (n, heads * head_dim)), _code(q, "q"),
+        _dev(v_cache, "v cache", q.dtype, (n_pages, kv_heads, value_dim, page_size) if v_transposed
+             else (n_pages, kv_heads, page_size, value_dim)),
+        _dev(out, "attention out", q.dtype, (n, heads * value_dim)), _code(q, "q"),
         _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
         _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size,
-        n, heads, kv_heads, head_dim, n_pages, float(scale), int(window or 0), int(v_transposed), _stream()),
-        "attention")
+        n, heads, kv_heads, head_dim, value_dim, n_pages, float(scale), int(window or 0), int(v_transposed),
+        _stream()), "attention")
     return out
 
 
@@ -738,4 +743,94 @@ def diff_attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
         _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size, n_rows, int(max_seg_len), heads,
         kv_heads, dim, vdim, n_pages, float(scale), int(window or 0), float(lam), float(eps), float(out_scale),
         int(min_len), _stream()), "diff_attention_tiles")
+    return out
+
+
+# ---------------------------------------------------------------- routed feed-forward, norm on a sublayer's result
+MOE_EPILOGUES = {None: 0, "none": 0, "relu2": 1}
+
+
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], choice: torch.Tensor, weight: torch.Tensor,
+              top: int) -> None:
+    """choice[t] = the `top` router outputs with the largest softmax(logits[t]) + correction, weight[t] their
+    softmax scores (as they are)."""
+    n, r = logits.shape
+    _check(library().imparo_moe_route(
+        _dev(logits, "router logits", torch.float32), _dev(correction, "router correction", torch.float32, (r,)),
+        _dev(choice, "choice", torch.int32, (n, top)), _dev(weight, "choice weights", torch.float32, (n, top)),
+        n, r, top, _stream()), "moe_route")
+
+
+def moe_tile_rows(n_entries: int, n_experts: int, dtype: torch.dtype) -> int:
+    return int(library().imparo_moe_tile_rows(int(n_entries), int(n_experts), 0 if dtype == torch.float32 else 1))
+
+
+def moe_max_tiles(n_entries: int, n_experts: int, tile_rows: int) -> int:
+    return int(library().imparo_moe_max_tiles(int(n_entries), int(n_experts), int(tile_rows)))
+
+
+def moe_plan(choice: torch.Tensor, n_experts: int, tile_rows: int, slot_of_entry: torch.Tensor,
+             entry_of_slot: torch.Tensor, tiles: torch.Tensor) -> None:
+    n_entries = choice.numel()
+    _dev(slot_of_entry, "slot_of_entry", torch.int32, (n_entries,))
+    _dev(entry_of_slot, "entry_of_slot", torch.int32, (n_entries,))
+    _check(library().imparo_moe_plan(
+        _dev(choice, "choice", torch.int32), n_entries, n_experts, tile_rows, slot_of_entry.data_ptr(),
+        entry_of_slot.data_ptr(), _dev(tiles, "tiles", torch.int32), tiles.shape[0], _stream()), "moe_plan")
+
+
+def moe_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, tiles: torch.Tensor, tile_rows: int,
+             entry_of_slot: Optional[torch.Tensor] = None, gather_div: int = 0, epilogue: Optional[str] = None) -> torch.Tensor:
+    """out[slot] = epilogue(a[row(slot)] . w[expert of the slot's tile]^T); w is [experts, n, k]."""
+    n_experts, n, k = w.shape
+    if a.dim() != 2 or a.shape[1] != k or a.dtype != w.dtype:
+        raise KernelArgumentError(f"moe_gemm: a is {tuple(a.shape)} {a.dtype}, the experts' matrices {tuple(w.shape)} {w.dtype}")
+    if out.dim() != 2 or out.shape[1] != n:
+        raise KernelArgumentError(f"moe_gemm: out is {tuple(out.shape)}, {n} columns are needed")
+    if gather_div == 0 and a.shape[0] < out.shape[0]:
+        raise KernelArgumentError("moe_gemm: fewer input rows than slots")
+    if epilogue not in MOE_EPILOGUES:
+        raise KernelArgumentError(f"moe_gemm: unknown epilogue {epilogue!r}")
+    if tiles.dim() != 2 or tiles.shape[1] != 3:
+        raise KernelArgumentError("moe_gemm: tiles is [max_tiles, 3]")
+    _check(library().imparo_moe_gemm(
+        _dev(a, "moe_gemm a"), a.stride(0), int(gather_div), _dev(entry_of_slot, "entry_of_slot", torch.int32),
+        _dev(w, "experts' matrices"), _dev(out, "moe_gemm out"), _code(out, "moe_gemm out"), _code(w, "experts' matrices"),
+        _dev(tiles, "tiles", torch.int32), tiles.shape[0], int(tile_rows), n, k, MOE_EPILOGUES[epilogue], _stream()),
+        "moe_gemm")
+    return out
+
+
+def moe_combine(y: torch.Tensor, h: torch.Tensor, choice: torch.Tensor, weight: torch.Tensor,
+                slot_of_entry: torch.Tensor, n_experts: int, out: torch.Tensor) -> torch.Tensor:
+    n, top = choice.shape
+    width = h.shape[1]
+    _check(library().imparo_moe_combine(
+        _dev(y, "experts' results", torch.float32), _dev(h, "feed-forward input", None, (n, width)), _code(h, "input"),
+        _dev(choice, "choice", torch.int32), _dev(weight, "choice weights", torch.float32, (n, top)),
+        _dev(slot_of_entry, "slot_of_entry", torch.int32, (n * top,)), _dev(out, "combined", torch.float32, (n, width)),
+        n, width, top, n_experts, _stream()), "moe_combine")
+    return out
+
+
+def post_norm_add(x: torch.Tensor, delta: torch.Tensor, w_post: torch.Tensor, eps_post: float,
+                  w_next: Optional[torch.Tensor] = None, eps_next: float = 0.0, out: Optional[torch.Tensor] = None,
+                  rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x += rms_norm(delta) * w_post (delta shaped like x, or [slices, *x.shape], added in order); with
+    `w_next`, out = rms_norm(x) * w_next. With `rows` only those rows are taken, into out, and x stays."""
+    n_x, width = x.shape
+    n_delta = delta.shape[0] if delta.dim() == 3 else 1
+    _dev(delta, "sublayer result", torch.float32, ((n_delta, n_x, width) if delta.dim() == 3 else (n_x, width)))
+    n_out = n_x if rows is None else rows.shape[0]
+    if w_next is not None:
+        if out is None or tuple(out.shape) != (n_out, width):
+            raise KernelArgumentError("post_norm_add: the next norm needs an output of one row per taken row")
+    elif rows is not None:
+        raise KernelArgumentError("post_norm_add: a row selection without a next norm has no result")
+    _check(library().imparo_post_norm_add(
+        _dev(x, "stream", torch.float32), delta.data_ptr(), n_delta, n_x, _dev(rows, "rows", torch.int32),
+        _dev(w_post, "post norm weight", torch.float32, (width,)), float(eps_post),
+        _dev(w_next, "next norm weight", torch.float32, (width,)), float(eps_next),
+        _dev(out, "normed") if w_next is not None else None, _code(out, "normed") if w_next is not None else 0,
+        n_out, width, _stream()), "post_norm_add")
     return out

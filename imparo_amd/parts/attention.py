@@ -5,7 +5,18 @@ and k, rotation, k and v appended to the cache at the tokens' positions before
 attention of the same batch, causal softmax attention bounded by position,
 then the output projection
 (/root/reference/crates/imparo-model/src/lfm2/workflow_cpu.rs:203-250,
-/root/reference/crates/imparo-model/src/cpu_support.rs:361-445)."""
+/root/reference/crates/imparo-model/src/cpu_support.rs:361-445).
+
+Parameters beyond the sizes: `value_dim` (a head's values where they are not
+head_dim wide), `window` (a query sees itself and the window - 1 positions
+before it), `keep_window` (what the cache keeps, where a layer that reads this
+layer's cache looks further back than this layer itself; None: everything),
+`shared_kv` (the layer has no key and value projections: it is run with
+another layer's cache, `LayerCall.cache_of`, and brings queries only),
+`weight_suffix` and `names` (how the checkpoint calls the tensors),
+`exact_weights` (the softmax weights stay float32 through the product with the
+values: the wave kernel instead of the matrix-core kernels, which round them
+to bfloat16)."""
 from __future__ import annotations
 
 from typing import Dict, Optional
@@ -17,7 +28,7 @@ from ..config.plan import PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .base import Declared, StepContext
-from .linear import Linear, place_matrix, place_vector
+from .linear import Linear, place_matrix, place_projection, place_vector
 from .registry import part_class, register_part
 
 _DEFAULT_NAMES = dict(q="q_proj", k="k_proj", v="v_proj", o="o_proj", q_norm="q_norm", k_norm="k_norm")
@@ -36,37 +47,48 @@ class Attention:
     @classmethod
     def declare(cls, spec: PartSpec) -> Declared:
         n = cls._names(spec)
+        sfx = spec.get("weight_suffix", ".weight")
         E, H, Hk, D = spec["width"], spec["heads"], spec["kv_heads"], spec["head_dim"]
-        out: Declared = {
-            n["q"] + ".weight": (TensorDecl((H * D, E)), "matrix"),
-            n["k"] + ".weight": (TensorDecl((Hk * D, E)), "matrix"),
-            n["v"] + ".weight": (TensorDecl((Hk * D, E)), "matrix"),
-            n["o"] + ".weight": (TensorDecl((E, H * D)), "matrix"),
-        }
+        Dv = spec.get("value_dim") or D
+        shared = bool(spec.get("shared_kv"))
+        out: Declared = {n["q"] + sfx: (TensorDecl((H * D, E)), "matrix"),
+                         n["o"] + sfx: (TensorDecl((E, H * Dv)), "matrix")}
+        if not shared:
+            out[n["k"] + sfx] = (TensorDecl((Hk * D, E)), "matrix")
+            out[n["v"] + sfx] = (TensorDecl((Hk * Dv, E)), "matrix")
         if spec.get("qk_norm") is not None:
-            out[n["q_norm"] + ".weight"] = (TensorDecl((D,), "vector"), "norm")
-            out[n["k_norm"] + ".weight"] = (TensorDecl((D,), "vector"), "norm")
+            out[n["q_norm"] + sfx] = (TensorDecl((D,), "vector"), "norm")
+            if not shared:
+                out[n["k_norm"] + sfx] = (TensorDecl((D,), "vector"), "norm")
         return out
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
                  engine_dtype: torch.dtype):
         n = self._names(spec)
+        sfx = spec.get("weight_suffix", ".weight")
         self.engine_dtype = engine_dtype
         self.v_transposed = False        # decided with the cache's page size, in cache_spec
         self.width, self.heads, self.kv_heads, self.head_dim = (spec["width"], spec["heads"], spec["kv_heads"],
                                                                 spec["head_dim"])
-        if self.head_dim % 16:
-            raise ValueError(f"attention kernels take head sizes in steps of 16, got {self.head_dim}")
+        self.value_dim = int(spec.get("value_dim") or self.head_dim)
+        self.shared_kv = bool(spec.get("shared_kv"))
+        self.exact_weights = bool(spec.get("exact_weights"))
+        if self.head_dim % 8:
+            raise ValueError(f"attention kernels take head sizes in steps of 8, got {self.head_dim}")
         if self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} heads cannot share {self.kv_heads} kv heads evenly")
         self.scale = float(spec["scale"])
         self.window: Optional[int] = spec.get("window")
-        ws = [tensors[n[x] + ".weight"] for x in ("q", "k", "v")]
+        self.keep_window: Optional[int] = spec.params["keep_window"] if "keep_window" in spec.params else self.window
+        ws = [tensors[n[x] + sfx] for x in (("q",) if self.shared_kv else ("q", "k", "v"))]
         if len({w.dtype for w in ws}) > 1:
             ws = [w.to(torch.float32) for w in ws]
         # one projection for q | k | v: the same dot products, one launch
-        self.qkv = Linear(place_matrix(torch.cat(ws, dim=0), engine_dtype, device))
-        self.out = Linear(place_matrix(tensors[n["o"] + ".weight"], engine_dtype, device))
+        self.qkv = Linear(place_projection(torch.cat(ws, dim=0), engine_dtype, device))
+        self.out = Linear(place_projection(tensors[n["o"] + sfx], engine_dtype, device))
+        if engine_dtype != torch.float32 and self.out.in_dtype == torch.float32:
+            raise ValueError(f"heads x value size = {self.heads * self.value_dim} must be a multiple of 8 under bfloat16 "
+                             f"(the attention kernels write their result in the cache's dtype)")
         norm = spec.get("qk_norm")
         if norm is not None:
             # the kernels that norm a head know one norm: RMS with a weight per dimension, no offset
@@ -74,8 +96,9 @@ class Attention:
                 raise ValueError(f"this attention mixer norms q and k per head with an RMS norm; the plan names "
                                  f"{norm.kind!r} (another norm on the heads is another mixer, with kernels of its own)")
             self.norm_eps = float(norm["eps"])
-            self.q_norm = place_vector(tensors[n["q_norm"] + ".weight"], device)
-            self.k_norm = place_vector(tensors[n["k_norm"] + ".weight"], device)
+            self.q_norm = place_vector(tensors[n["q_norm"] + sfx], device)
+            # a layer without keys of its own hands the kernels its query weight in the key weight's place
+            self.k_norm = self.q_norm if self.shared_kv else place_vector(tensors[n["k_norm"] + sfx], device)
         else:
             self.norm_eps, self.q_norm, self.k_norm = 0.0, None, None
         pos = spec.get("position") or PartSpec("none")
@@ -91,8 +114,9 @@ class Attention:
         """Keys and values per position, laid out as this mixer's kernels read
         them: where the matrix-core kernels apply (bfloat16, pages of at least
         16, head sizes up to 128), V is kept transposed inside a page."""
-        self.v_transposed = ops.mfma_attention_supported(self.engine_dtype, page_size, self.head_dim)
-        return kv_spec(self.kv_heads, self.head_dim, self.window, self.v_transposed)
+        self.v_transposed = (self.value_dim == self.head_dim and not self.exact_weights
+                             and ops.mfma_attention_supported(self.engine_dtype, page_size, self.head_dim))
+        return kv_spec(self.kv_heads, self.head_dim, self.keep_window, self.v_transposed, self.value_dim)
 
     def _portion_tiles(self, ctx: StepContext) -> int:
         """Tiles of queries that the portions of this batch make, as the prompt kernel counts them."""
@@ -113,12 +137,15 @@ class Attention:
 
     def forward(self, ctx: StepContext, site: int, owns_cache: bool, h: torch.Tensor) -> torch.Tensor:
         T = h.shape[0]
+        if self.shared_kv and owns_cache:
+            raise ValueError("a layer without key and value projections must be run with another layer's cache")
         qkv = self.qkv(ctx, h, torch.float32, "qkv", alias="mixer_in")
         k_cache, v_cache, table = ctx.kv(site)
         vt = self.v_transposed
         inv_freq = self.position.inv_freq
         interleaved = bool(getattr(self.position, "interleaved", False))
-        if (vt and owns_cache and ctx.single_rows is not None and ctx.n_single_rows == T and not ctx.n_portion_rows
+        Dv = self.value_dim
+        if (vt and owns_cache and Dv == self.head_dim and ctx.single_rows is not None and ctx.n_single_rows == T and not ctx.n_portion_rows
                 and ops.attention_decode_qkv_pays(T, ctx.max_context)
                 and ops.attention_decode_qkv_takes(self.head_dim, 0 if inv_freq is None else inv_freq.shape[0])):
             # every row brings one token: head norm, rotation and the write of the new key and value ride
@@ -134,8 +161,9 @@ class Attention:
         ops.qk_norm_rope_store(qkv, self.q_norm, self.k_norm, self.norm_eps, inv_freq,
                                ctx.positions, ctx.row_of_token, table if owns_cache else None, ctx.page_size,
                                q, k_cache if owns_cache else None, v_cache if owns_cache else None,
-                               self.heads, self.kv_heads, self.head_dim, v_transposed=vt, interleaved=interleaved)
-        o = ctx.workspace.get("attn_out", (T, self.heads * self.head_dim), ctx.dtype, alias="mixer_mid")
+                               self.heads, 0 if self.shared_kv else self.kv_heads, self.head_dim, v_transposed=vt,
+                               interleaved=interleaved, value_dim=Dv)
+        o = ctx.workspace.get("attn_out", (T, self.heads * Dv), ctx.dtype, alias="mixer_mid")
         if vt and ctx.single_rows is not None:
             # matrix-core kernels: single tokens split over their keys, portions tiled over their queries
             if ctx.n_single_rows:
@@ -164,6 +192,10 @@ class Attention:
         # a delta for the residual stream: the next norm adds slices, so it may come sliced
         return self.out(ctx, o, torch.float32, "mixer_out", sliced_ok=True, into=ctx.stream)
 
+
+    def can_emit(self) -> bool:
+        # the step program's attention has one head size, keys and values of its own, and the matrix-core kernels
+        return self.value_dim == self.head_dim and not self.shared_kv and not self.exact_weights
 
     def emit(self, program, site: int, owns_cache: bool) -> None:
         """Appends `forward` to a native step program."""

@@ -148,3 +148,6 @@ class Residual:
     inner dimension, which the norm adds up in order."""
     x: torch.Tensor
     pending: Optional[torch.Tensor] = None
+    # (weight, eps) of an RMS norm that the pending delta goes through before it is added (a block that
+    # norms what its sublayers return); the norm that adds the delta applies it in the same launch
+    post: Optional[Tuple[torch.Tensor, float]] = None

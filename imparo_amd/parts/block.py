@@ -83,4 +83,31 @@ class PreNormBlock:
         return None if delta is res.x else delta
 
 
+class SandwichBlock(PreNormBlock):
+    """x += post_a(mixer(norm_a(x))); x += post_b(ffn(norm_b(x))): a norm before and behind each
+    sublayer. The parts `mixer_post` and `ffn_post` are norms (their weights may carry a layer
+    scale and a residual multiplier); a sublayer's result is left pending on the stream together
+    with its norm, and the next norm that reads the stream, whichever block it belongs to, applies
+    that norm, adds and norms the sum in one launch."""
+
+    def __init__(self, parts: Dict[str, object]):
+        super().__init__(parts)
+        if self.shift is not None:
+            raise ValueError("this arrangement has no token shift")
+        self.mixer_post, self.ffn_post = parts["mixer_post"], parts.get("ffn_post")
+        if (self.ffn is None) != (self.ffn_post is None):
+            raise ValueError("a block has a feed-forward and the norm behind it, or neither")
+
+    def forward(self, ctx: StepContext, res: Residual, site: int, owns_cache: bool) -> None:
+        h = self.mixer_norm.forward(ctx, res, self.mixer.in_dtype)
+        res.pending, res.post = self.mixer.forward(ctx, site, owns_cache, h), self.mixer_post.as_post()
+        if self.ffn is not None:
+            n = self.ffn_norm.forward(ctx, res, self.ffn.in_dtype)
+            res.pending, res.post = self.ffn.forward(ctx, n), self.ffn_post.as_post()
+
+    def can_emit(self) -> bool:
+        return False          # the step program knows the pre-norm block only
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "sandwich", SandwichBlock)

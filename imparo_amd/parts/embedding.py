@@ -1,4 +1,4 @@
-"""Token embedding (a row gather, no scale:
+"""Token embedding (a row gather; `scale` multiplies the row in float32, 1 in the reference:
 /root/reference/crates/imparo-model/src/cpu_support.rs:327-342) and the output
 head (logits = W h for the rows that want logits, no bias, no softcap:
 /root/reference/crates/imparo-model/src/cpu_support.rs:451-466).
@@ -41,10 +41,14 @@ class Embedding:
             placed[name] = place_matrix(tensors[name], engine_dtype, device)
         self.table = placed[name]
         self.vocab, self.width = spec["vocab"], spec["width"]
+        self.scale = float(spec.get("scale", 1.0))
 
     def forward(self, ctx: StepContext, token_ids: torch.Tensor) -> torch.Tensor:
         x = ctx.workspace.get("residual", (token_ids.shape[0], self.width), torch.float32)
-        return ops.embed_gather(self.table, token_ids, x)
+        return ops.embed_gather(self.table, token_ids, x, self.scale)
+
+    def can_emit(self) -> bool:
+        return self.scale == 1.0          # the step program's gather has no scale
 
     def emit(self, program) -> None:
         """Appends `forward` to a native step program."""

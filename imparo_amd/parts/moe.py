@@ -1,0 +1,115 @@
+"""A routed feed-forward: a mixture of small feed-forward layers (experts) of
+which every token uses a few.
+
+Router: z = Wr n in float32; scores s = softmax(z) over all router outputs;
+the `top` outputs with the largest s + correction are chosen (the correction
+moves the choice only) and their weights are their scores s, as they are, not
+renormalized. The first `experts` router outputs are real experts,
+y = Wdown act(Wup n) without biases; the last `identity` outputs stand for
+experts that pass their input through. The result is the weighted sum of the
+chosen experts' outputs, added in the order of the choice.
+
+Parameters: width, hidden (an expert's), experts, identity, top, activation
+("relu2": the square of max(z, 0)), and the tensors' names: `router`,
+`correction` (None: no correction), `expert_up` / `expert_down` as patterns
+with `{e}` for the expert's number.
+
+The experts' matrices lie stacked, [experts, out, in]. A step sorts its (token,
+choice) entries by expert on the device and runs the two products over tiles of
+one expert's rows each; the grids are sized by a bound the host knows, so
+nothing comes back to the host and a step of this part can be captured.
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..config.plan import PartSpec
+from ..kernels import ops
+from ..weights.loader import TensorDecl
+from .base import Declared, StepContext
+from .linear import Linear, place_matrix, place_projection, place_vector
+from .registry import register_part
+
+
+class RoutedExperts:
+    role = "feed_forward"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
+
+    @staticmethod
+    def _names(spec: PartSpec) -> Dict[str, str]:
+        names = dict(router="router", correction="correction", expert_up="e{e}.up", expert_down="e{e}.down")
+        names.update(spec.get("names") or {})
+        return {k: (None if v is None else f"{spec.prefix}.{v}") for k, v in names.items()}
+
+    @classmethod
+    def declare(cls, spec: PartSpec) -> Declared:
+        n = cls._names(spec)
+        E, F, X, I = spec["width"], spec["hidden"], spec["experts"], spec.get("identity", 0)
+        out: Declared = {n["router"]: (TensorDecl((X + I, E)), "matrix")}
+        if n["correction"] is not None:
+            out[n["correction"]] = (TensorDecl((X + I,), "vector"), "bias")
+        for e in range(X):
+            out[n["expert_up"].format(e=e)] = (TensorDecl((F, E)), "matrix")
+            out[n["expert_down"].format(e=e)] = (TensorDecl((E, F)), "matrix")
+        return out
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
+                 engine_dtype: torch.dtype):
+        n = self._names(spec)
+        self.width, self.hidden = spec["width"], spec["hidden"]
+        self.experts, self.identity, self.top = spec["experts"], int(spec.get("identity", 0)), spec["top"]
+        self.activation = spec.get("activation", "relu2")
+        if self.activation not in ops.MOE_EPILOGUES or self.activation in (None, "none"):
+            raise ValueError(f"the experts' activation {self.activation!r} is not one the product's epilogue knows")
+        if not 1 <= self.top <= self.experts + self.identity:
+            raise ValueError(f"{self.top} of {self.experts + self.identity} experts cannot be chosen")
+        # bfloat16 x bfloat16 products are exact in float32 and the sums are float32: the router runs in 32 bits
+        # on the matrix cores too; its input is the norm's output in the engine's dtype
+        self.router = Linear(place_projection(tensors[n["router"]], engine_dtype, device))
+        self.correction = None if n["correction"] is None else place_vector(tensors[n["correction"]], device)
+        ups = [tensors[n["expert_up"].format(e=e)] for e in range(self.experts)]
+        downs = [tensors[n["expert_down"].format(e=e)] for e in range(self.experts)]
+        if self.experts:
+            up, down = torch.stack(ups), torch.stack(downs)
+            # The bfloat16 products walk K in steps of 8: a hidden width that is no multiple of 8 is filled up
+            # with hidden units of zero weight (act(0) = 0 goes through zero columns of the way back).
+            fill = (-self.hidden) % 8
+            if fill and engine_dtype != torch.float32:
+                up = torch.cat([up, up.new_zeros(self.experts, fill, self.width)], dim=1)
+                down = torch.cat([down, down.new_zeros(self.experts, self.width, fill)], dim=2)
+            if engine_dtype != torch.float32 and (self.width % 8 or self.router.in_dtype == torch.float32):
+                up, down = up.to(torch.float32), down.to(torch.float32)      # such a width runs in float32 throughout
+            self.up = place_matrix(up, engine_dtype, device)
+            self.down = place_matrix(down, engine_dtype, device)
+        else:
+            self.up = self.down = None
+
+    @property
+    def in_dtype(self) -> torch.dtype:
+        return self.router.in_dtype
+
+    def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
+        T, top, X = n.shape[0], self.top, self.experts
+        ws = ctx.workspace
+        z = self.router(ctx, n, torch.float32, "router_logits")
+        choice = ws.get("moe_choice", (T, top), torch.int32)
+        weight = ws.get("moe_weight", (T, top), torch.float32)
+        ops.moe_route(z, self.correction, choice, weight, top)
+        entries = T * top
+        slot_of_entry = ws.get("moe_slot_of_entry", (entries,), torch.int32)
+        y = ws.get("moe_y", (entries, self.width), torch.float32)
+        if X:
+            rows = ops.moe_tile_rows(entries, X, self.up.dtype)
+            tiles = ws.get("moe_tiles", (ops.moe_max_tiles(entries, X, rows), 3), torch.int32)
+            entry_of_slot = ws.get("moe_entry_of_slot", (entries,), torch.int32)
+            ops.moe_plan(choice, X, rows, slot_of_entry, entry_of_slot, tiles)
+            hidden = ws.get("moe_hidden", (entries, self.up.shape[1]), self.up.dtype, alias="mixer_in")
+            ops.moe_gemm(n, self.up, hidden, tiles, rows, entry_of_slot, gather_div=top, epilogue=self.activation)
+            ops.moe_gemm(hidden, self.down, y, tiles, rows)
+        out = ws.get("ffn_out", (T, self.width), torch.float32)
+        return ops.moe_combine(y, n, choice, weight, slot_of_entry, X, out)
+
+
+register_part("feed_forward", "routed_experts", RoutedExperts)

@@ -6,7 +6,15 @@ precedes a norm is fused into it (the reference's add_rms_norm,
 With `groups` > 1 the row is cut into that many equal consecutive parts and
 each is divided by its own root mean square; the weight spans the whole row.
 `tensor` names the weight outright where a checkpoint does not call it
-`<prefix>.weight`."""
+`<prefix>.weight`. `offset` is added to the stored weight (1 for a weight kept
+around zero). `scale_tensor` names a second vector of the row's width and
+`multiplier` a constant that the normed row is multiplied by as well (a layer
+scale and a residual multiplier on a norm that sits behind a sublayer): all
+three are folded into one float32 weight when the model is loaded.
+
+A block may leave its sublayer's result pending on the stream together with
+the norm it goes through before the add (`Residual.post`); this norm then
+applies that norm, adds, and norms the sum in one launch."""
 from __future__ import annotations
 
 from typing import Dict
@@ -31,7 +39,11 @@ class RmsNorm:
 
     @classmethod
     def declare(cls, spec: PartSpec) -> Declared:
-        return {cls._tensor(spec): (TensorDecl((spec["width"],), "vector"), "norm")}
+        # a weight that an offset of 1 is added to is stored around zero
+        out = {cls._tensor(spec): (TensorDecl((spec["width"],), "vector"), "bias" if spec.get("offset") else "norm")}
+        if spec.get("scale_tensor"):
+            out[spec["scale_tensor"]] = (TensorDecl((spec["width"],), "vector"), "norm")
+        return out
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
                  engine_dtype: torch.dtype):
@@ -40,14 +52,30 @@ class RmsNorm:
         self.groups = int(spec.get("groups") or 1)
         if self.groups < 1 or self.width % self.groups:
             raise ValueError(f"a norm over {self.width} values cannot be cut into {self.groups} equal parts")
-        self.weight = place_vector(tensors[self._tensor(spec)], device)
+        weight = tensors[self._tensor(spec)].to(torch.float32) + float(spec.get("offset") or 0.0)
+        if spec.get("scale_tensor"):
+            weight = weight * tensors[spec["scale_tensor"]].to(torch.float32)
+        if spec.get("multiplier") is not None:
+            weight = weight * float(spec["multiplier"])
+        self.weight = place_vector(weight, device)
+
+    def as_post(self):
+        """(weight, eps) for `Residual.post`: this norm applied to a sublayer's result by whoever adds it."""
+        if self.groups != 1:
+            raise ValueError("a norm behind a sublayer does not cut rows into groups")
+        return self.weight, self.eps
 
     def forward(self, ctx: StepContext, res: Residual, out_dtype: torch.dtype, name: str = "normed") -> torch.Tensor:
         """Adds the pending delta into the stream (if any) and returns the
         normed rows in `out_dtype`."""
         out = ctx.workspace.get(name, tuple(res.x.shape), out_dtype)
         pending, res.pending = res.pending, None
-        if self.groups > 1:
+        post, res.post = res.post, None
+        if post is not None and pending is not None:
+            if self.groups > 1:
+                raise ValueError("a norm in groups cannot take a sublayer's result through a norm of its own")
+            ops.post_norm_add(res.x, pending, post[0], post[1], self.weight, self.eps, out)
+        elif self.groups > 1:
             ops.group_rms_norm(res.x, self.weight, self.groups, self.eps, out, delta=pending,
                                write_back=pending is not None)
         elif pending is not None:
@@ -61,6 +89,8 @@ class RmsNorm:
         """`forward` for a step whose rows all bring one token, with the token shift behind the norm in
         the same launch: out = h + (prev - h) * mix, where the request's prev (state[slot]) becomes h."""
         out = ctx.workspace.get(name, tuple(res.x.shape), out_dtype)
+        if res.post is not None:
+            raise ValueError("the norm with the token shift does not take a sublayer's result through a norm of its own")
         pending, res.pending = res.pending, None
         ops.group_rms_norm(res.x, self.weight, self.groups, self.eps, out, delta=pending,
                            write_back=pending is not None, shift_mix=mix, shift_state=state, slot=ctx.slot)
@@ -84,7 +114,11 @@ class RmsNorm:
         """Norm of selected rows only (the rows whose logits are wanted); the
         stream itself is left as it is."""
         out = ctx.workspace.get(name, (rows.shape[0], self.width), out_dtype)
-        if self.groups > 1:
+        if res.post is not None and res.pending is not None:
+            if self.groups > 1:
+                raise ValueError("a norm in groups cannot take a sublayer's result through a norm of its own")
+            ops.post_norm_add(res.x, res.pending, res.post[0], res.post[1], self.weight, self.eps, out, rows=rows)
+        elif self.groups > 1:
             ops.group_rms_norm(res.x, self.weight, self.groups, self.eps, out, delta=res.pending, rows=rows)
         else:
             ops.rms_norm(res.x, self.weight, self.eps, out, delta=res.pending, rows=rows)
