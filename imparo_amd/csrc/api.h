@@ -82,7 +82,7 @@ int imparo_attention(const void* q, const void* k_cache, const void* v_cache, vo
 
 // The two above for heads whose values have another size than their keys (value_dim): a token's row is
 // heads + kv_heads units of head_dim, then kv_heads units of value_dim; the value cache holds value_dim a
-// position and out is [tokens, heads * value_dim]. head_dim a multiple of 8. The store also takes rows of
+// position and out is [tokens, heads * value_dim]; any head_dim up to 512. The store also takes rows of
 // queries only (kv_heads 0, write_kv 0), for a layer that reads another layer's keys and values.
 int imparo_qk_norm_rope_store_dv(const float* qkv, const float* q_weight, const float* k_weight, float eps,
                                  const float* inv_freq, int n_freq, int interleaved,

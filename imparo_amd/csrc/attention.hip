@@ -46,6 +46,14 @@ __device__ __forceinline__ float dot_row<bf16_t>(const float* __restrict__ q, co
     return s;
 }
 
+// a head size that is no multiple of a 16-byte vector: element by element, in the same order
+template <typename T>
+__device__ __forceinline__ float dot_row_any(const float* __restrict__ q, const T* __restrict__ k, int head_dim) {
+    float s = 0.f;
+    for (int i = 0; i < head_dim; ++i) s += q[i] * load_f32<T>(k, i);
+    return s;
+}
+
 template <typename T>
 __global__ void k_attention_wave(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                  T* __restrict__ out, const int32_t* __restrict__ positions,
@@ -86,7 +94,8 @@ __global__ void k_attention_wave(const T* __restrict__ q, const T* __restrict__ 
             const int page = table[p / page_size];
             if (page >= 0 && page < n_pages) {
                 off = (((long long)page * kv_heads + kvh) * page_size + (p % page_size)) * head_dim;
-                s = dot_row<T>(qr, k_cache + off, head_dim) * scale;
+                s = (head_dim % Vec16<T>::N == 0 ? dot_row<T>(qr, k_cache + off, head_dim)
+                                                 : dot_row_any<T>(qr, k_cache + off, head_dim)) * scale;
                 // from here on `off` is where the key's value row starts
                 off = v_transposed ? ((long long)page * kv_heads + kvh) * page_size * value_dim + (p % page_size)
                                    : (((long long)page * kv_heads + kvh) * page_size + (p % page_size)) * value_dim;
@@ -131,7 +140,7 @@ static int check_attention_args(const void* q, const void* k_cache, const void* 
                                 int n_pages, int window) {
     if (!q || !k_cache || !v_cache || !out || !positions || !row_of_token || !block_table) return IMPARO_BAD_ARGUMENT;
     if (n_tokens < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0) return IMPARO_BAD_ARGUMENT;
-    if (head_dim <= 0 || head_dim % 8 != 0 || head_dim > ATT_MAX_HEAD_DIM) return IMPARO_BAD_ARGUMENT;
+    if (head_dim <= 0 || head_dim > ATT_MAX_HEAD_DIM) return IMPARO_BAD_ARGUMENT;
     if (page_size <= 0 || table_stride <= 0 || n_pages <= 0 || window < 0) return IMPARO_BAD_ARGUMENT;
     return IMPARO_OK;
 }

@@ -221,15 +221,13 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_we
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
               positions: torch.Tensor, row_of_token: torch.Tensor, block_table: torch.Tensor,
               scale: float, window: Optional[int], v_transposed: bool = False) -> torch.Tensor:
-    """The general kernel: any page size, head sizes in steps of 16 up to 512,
-    float32 or bfloat16; one wave per (token, head)."""
+    """The general kernel: any page size, head sizes up to 512 (values of a size of their own
+    are read off the value cache's shape), float32 or bfloat16; one wave per (token, head)."""
     n, heads, head_dim = q.shape
     n_pages, kv_heads, page_size, hd = k_cache.shape
     value_dim = v_cache.shape[2] if v_transposed else v_cache.shape[3]
     if hd != head_dim:
         raise KernelArgumentError(f"attention: q has head size {head_dim}, the cache {hd}")
-    if head_dim % 8 != 0:
-        raise KernelArgumentError(f"attention: head size must be a multiple of 8, got {head_dim}")
     if heads % kv_heads != 0:
         raise KernelArgumentError(f"attention: {heads} heads cannot share {kv_heads} kv heads evenly")
     _check(library().imparo_attention_dv(

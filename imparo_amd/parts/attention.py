@@ -73,8 +73,6 @@ class Attention:
         self.value_dim = int(spec.get("value_dim") or self.head_dim)
         self.shared_kv = bool(spec.get("shared_kv"))
         self.exact_weights = bool(spec.get("exact_weights"))
-        if self.head_dim % 8:
-            raise ValueError(f"attention kernels take head sizes in steps of 8, got {self.head_dim}")
         if self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} heads cannot share {self.kv_heads} kv heads evenly")
         self.scale = float(spec["scale"])

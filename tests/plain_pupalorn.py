@@ -157,3 +157,13 @@ class PlainPupalorn:
             if layers_out is not None:
                 layers_out.append(x.clone())
         return offset_norm(x, w["final.norm"], eps) @ w["head"].T
+
+    def logits(self, tokens: List[int], order=None) -> torch.Tensor:
+        return self.forward(list(tokens)).to(torch.float32)
+
+    def greedy(self, prompt: List[int], n: int) -> List[int]:
+        tokens, out = list(prompt), []
+        for _ in range(n):
+            out.append(int(self.forward(tokens)[-1].argmax()))
+            tokens.append(out[-1])
+        return out
