@@ -402,20 +402,34 @@ def tumadra_shape(width, heads, kv_heads, ff, inner, layers=16, attention_at=(2,
                              mixer=attention if i in attention_at else scan, mlp=mlp) for i in range(layers)])
 
 
-def tumadra_workload(dtype, steps, warmup):
-    """Prefill and decode throughput of the Tumadra design at two sizes, beside LFM2 (the closest model
-    the engine has: a hybrid of attention and a fixed-state mixer) at equal size, through the same loops."""
+def pupalorn_shape(width, heads, kv_heads, expert_ff, experts=8, top=4, identity=2, layers=16, window=4096):
+    """A Pupalorn model with the attention sizes of the LFM2 shapes above (heads of 64, rotated whole) in every
+    layer, every second layer reading the keys and values of the layer before it, windows as long as the
+    benchmark's contexts (every cached key is read, as in LFM2's attention), and a mixture of experts whose
+    `top` chosen experts together are as wide as the LFM2 shape's feed-forward."""
+    def mixer(i):
+        m = dict(heads=heads, kv_heads=kv_heads, dim=64, vdim=64, scale=0.125, mask=dict(size=window),
+                 rot=dict(dims=64, base=1000000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
+        if i % 2:
+            m["kv_from"] = i - 1
+        return m
+    mlp = dict(kind="moe", expert=dict(ff=expert_ff), router=dict(experts=experts, identity=identity, top=top))
+    return dict(architecture="Pupalorn", vocab=65536, width=width, norm=dict(eps=1e-5), residual_mult=0.5,
+                embedding=dict(scale=1.0), layers=[dict(type="attention", mixer=mixer(i), mlp=mlp) for i in range(layers)])
+
+
+def compare_workload(workload, sizes, dtype, steps, warmup):
+    """Prefill and decode throughput of one design at some sizes, beside LFM2 (the closest model the engine
+    has) at equal layer sizes, through the same loops. `sizes`: (name, LFM2 configuration, the design's)."""
     import torch
     from imparo_amd.engine.model import declared_tensors
     from imparo_amd.sampling import Sampler
-    sizes = [
-        ("1.2B", LFM2_1_2B, tumadra_shape(2048, 16, 4, 12288, 2816)),
-        ("350M", LFM2_350M, tumadra_shape(1024, 8, 4, 6912, 1408)),
-    ]
-    out = {"workload": "tumadra", "dtype": dtype, "data": "synthetic token ids, random weights", "sizes": []}
-    for name, lfm2, tumadra in sizes:
+    out = {"workload": workload, "dtype": dtype, "data": "synthetic token ids, random weights", "sizes": []}
+    for name, lfm2, other in sizes:
         row = {"size": name}
-        for label, cfg in (("lfm2", lfm2), ("tumadra", tumadra)):
+        for label, cfg in (("lfm2", lfm2), (workload, other)):
+            if cfg is None:
+                continue
             print(f"[bench] {name} {label}: writing random weights ...", file=sys.stderr, flush=True)
             engine = build_engine(cfg, 2, dtype, max_tokens=8 * (4096 + 64) + 8192 + 64, max_requests=8,
                                   max_step_tokens=8192)
@@ -434,11 +448,31 @@ def tumadra_workload(dtype, steps, warmup):
             row[label] = r
             del engine, sampler
             torch.cuda.empty_cache()
-        for key in list(row["tumadra"]):
-            if key.endswith("tok_s"):
-                row.setdefault("tumadra_over_lfm2", {})[key] = round(row["tumadra"][key] / row["lfm2"][key], 3)
+        if "lfm2" in row and workload in row:
+            for key in list(row[workload]):
+                if key.endswith("tok_s"):
+                    row.setdefault(f"{workload}_over_lfm2", {})[key] = round(row[workload][key] / row["lfm2"][key], 3)
         out["sizes"].append(row)
     return out
+
+
+def tumadra_workload(dtype, steps, warmup):
+    """The Tumadra design at two sizes beside LFM2 (a hybrid of attention and a fixed-state mixer, as it is)."""
+    return compare_workload("tumadra", [
+        ("1.2B", LFM2_1_2B, tumadra_shape(2048, 16, 4, 12288, 2816)),
+        ("350M", LFM2_350M, tumadra_shape(1024, 8, 4, 6912, 1408)),
+    ], dtype, steps, warmup)
+
+
+def pupalorn_workload(dtype, steps, warmup, only=None, alone=False):
+    """The Pupalorn design at two sizes beside LFM2 (whose attention layers are the same mechanism: grouped
+    queries, per-head norms, rotation, the paged cache). `only`: one size; `alone`: without the LFM2 runs."""
+    sizes = [
+        ("1.2B", LFM2_1_2B, pupalorn_shape(2048, 32, 8, 2048)),
+        ("350M", LFM2_350M, pupalorn_shape(1024, 16, 8, 1152)),
+    ]
+    sizes = [(n, None if alone else a, b) for n, a, b in sizes if only in (None, n)]
+    return compare_workload("pupalorn", sizes, dtype, steps, warmup)
 
 
 def main() -> int:
@@ -452,11 +486,14 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="run only the 2,048-token prefill (for profiling)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "long", "tumadra"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "long", "tumadra", "pupalorn"],
                     help="decode: the headline line (default). serving: continuous batching of 32 requests in 4 "
                          "waves (LFM2-700M shape). long: 64 requests of 32,768-token prompts, then 128 tokens "
                          "each (LFM2-350M shape). tumadra: prefill and decode of the Tumadra design at two sizes "
-                         "beside LFM2 at equal size. The last three print a line of their own")
+                         "beside LFM2 at equal size; pupalorn: the same for the Pupalorn design. The last four "
+                         "print a line of their own")
+    ap.add_argument("--size", default=None, choices=["1.2B", "350M"], help="--workload pupalorn: one size only")
+    ap.add_argument("--alone", action="store_true", help="--workload pupalorn: without the LFM2 runs beside it")
     ap.add_argument("--requests", type=int, default=64, help="--workload long: concurrent requests")
     ap.add_argument("--prompt-len", type=int, default=32768, help="--workload long: tokens per prompt")
     ap.add_argument("--portion", type=int, default=2048, help="--workload long: tokens of a prompt per step")
@@ -472,6 +509,9 @@ def main() -> int:
         return 0
     if args.workload == "tumadra":
         print(json.dumps(tumadra_workload(args.dtype, args.steps, args.warmup)), flush=True)
+        return 0
+    if args.workload == "pupalorn":
+        print(json.dumps(pupalorn_workload(args.dtype, args.steps, args.warmup, args.size, args.alone)), flush=True)
         return 0
 
     import torch

@@ -80,6 +80,24 @@ int imparo_attention(const void* q, const void* k_cache, const void* v_cache, vo
                      int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
                      float scale, int window, int v_transposed, imparo_stream stream);
 
+// imparo_attention_decode and imparo_attention_prefill (below) with the softmax weights kept to float32
+// through the product with the values: a weight goes in as its bfloat16 rounding plus, through a second
+// product, the bfloat16 rounding of what that took off (16 bits of mantissa and more), and the
+// denominator sums the weights as they are. Same arguments.
+int imparo_attention_decode_exact(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                  float* part_o, float* part_ml, const int32_t* rows, int n_rows,
+                                  const int32_t* seg_start, const int32_t* positions,
+                                  const int32_t* block_table, int table_stride, int page_size,
+                                  int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                                  int n_splits, imparo_stream stream);
+int imparo_attention_prefill_exact(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                   float* part_o, float* part_ml, int n_splits,
+                                   const int32_t* rows, int n_rows, int n_tiles,
+                                   const int32_t* seg_start, const int32_t* seg_len, const int32_t* positions,
+                                   const int32_t* block_table, int table_stride, int page_size,
+                                   int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                                   imparo_stream stream);
+
 // The two above for heads whose values have another size than their keys (value_dim): a token's row is
 // heads + kv_heads units of head_dim, then kv_heads units of value_dim; the value cache holds value_dim a
 // position and out is [tokens, heads * value_dim]; any head_dim up to 512. The store also takes rows of

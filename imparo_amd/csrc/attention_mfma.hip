@@ -120,7 +120,8 @@ __device__ __forceinline__ void decode_load(DecodeTile<ND>& r, const Paged& kv, 
 // lane's query. `full`: every key of the tile is inside every query's range.
 template <int ND>
 __device__ __forceinline__ void decode_tile(DecodeState<ND>& st, const DecodeTile<ND>& r, int key_base, int lo_q,
-                                            int hi_q, int lo_all, int hi_all, bool full, float scale, int lane) {
+                                            int hi_q, int lo_all, int hi_all, bool full, float scale, int lane,
+                                            bool exact = false) {
     constexpr int D = ND * 16, NK = (ND + 1) / 2;
     const int g = lane >> 4;
     // ---- scores of keys kg .. kg+7: sv[4*t + i] from product t, row 4*g + i
@@ -152,13 +153,17 @@ __device__ __forceinline__ void decode_tile(DecodeState<ND>& st, const DecodeTil
         uint4 u;
         bf16x8 v;
         bf16_t h[8];
-    } pb;
+    } pb, pl;
     float psum = 0.f;
+    pl.u = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const float p = (sv[j] == -INFINITY) ? 0.f : __expf(sv[j] - m_new);
         pb.h[j] = f32_to_bf16(p);
-        psum += bf16_to_f32(pb.h[j]);             // the denominator sums what the product uses
+        // `exact`: what the rounding to bfloat16 took off a weight goes through a second product, so the
+        // weights meet the values with 16 bits of mantissa and more, and the denominator sums them as they are
+        if (exact) pl.h[j] = f32_to_bf16(p - bf16_to_f32(pb.h[j]));
+        psum += exact ? p : bf16_to_f32(pb.h[j]);             // the denominator sums what the product uses
     }
     psum += __shfl_xor(psum, 16, WAVE);
     psum += __shfl_xor(psum, 32, WAVE);
@@ -180,6 +185,7 @@ __device__ __forceinline__ void decode_tile(DecodeState<ND>& st, const DecodeTil
         }
         st.o[dt] = st.o[dt] * corr;
         st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb.v, st.o[dt], 0, 0, 0);
+        if (exact) st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pl.v, st.o[dt], 0, 0, 0);
     }
 }
 
@@ -285,7 +291,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 4 : 2) void k_attn_decod
     float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ seg_start, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
-    float scale, int window, int n_splits, FromQkv fq) {
+    float scale, int window, int n_splits, FromQkv fq, int exact) {
     constexpr int D = ND * 16, NK = (ND + 1) / 2;
     constexpr int TILES = DEC_SPLIT / (MFMA_WAVES * 32);   // tiles a wave takes at most
     __shared__ float sm[MFMA_WAVES][16], sl[MFMA_WAVES][16];
@@ -359,7 +365,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 4 : 2) void k_attn_decod
         const int kb = k_begin + (wave + j * MFMA_WAVES) * 32;
         if (kb < k_end) {
             const bool full = kb >= lo && kb + 31 <= last;
-            decode_tile<ND>(st, regs[j], kb, lo, hi_q, lo, last, full, scale, lane);
+            decode_tile<ND>(st, regs[j], kb, lo, hi_q, lo, last, full, scale, lane, exact != 0);
         }
     }
     if constexpr (FROM_QKV) {
@@ -560,7 +566,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     bf16_t* __restrict__ out, const int32_t* __restrict__ rows, int n_rows,
     const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
-    float scale, int window) {
+    float scale, int window, int exact) {
     constexpr int D = ND * 16;
     constexpr int LDK = PF_LD_K(D);
     const int page_shift = __ffs(page_size) - 1;          // a power of two: divisions by it are shifts
@@ -709,22 +715,27 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
             const float m_new = fmaxf(st.m, mx);
             const float corr = (st.m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(st.m - m_new);
             const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;        // exp2(-inf - 0) = 0: masked keys
-            s16x4 pb[4];
+            s16x4 pb[4], pl[4];
             float psum = 0.f;
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt) {
                 union {
                     uint32_t u[2];
                     s16x4 v;
-                } pk;
+                } pk, lo;
+                lo.u[0] = lo.u[1] = 0u;
 #pragma unroll
                 for (int i = 0; i < 4; i += 2) {
                     const float p0 = __builtin_amdgcn_exp2f(sc[kt][i] - m_sub), p1 = __builtin_amdgcn_exp2f(sc[kt][i + 1] - m_sub);
                     pk.u[i >> 1] = f32x2_to_bf16x2(p0, p1);
+                    const float h0 = __uint_as_float(pk.u[i >> 1] << 16), h1 = __uint_as_float(pk.u[i >> 1] & 0xffff0000u);
+                    // `exact`: what the rounding took off a weight goes through a second product
+                    if (exact) lo.u[i >> 1] = f32x2_to_bf16x2(p0 - h0, p1 - h1);
                     // the denominator sums what the product uses
-                    psum += __uint_as_float(pk.u[i >> 1] << 16) + __uint_as_float(pk.u[i >> 1] & 0xffff0000u);
+                    psum += exact ? p0 + p1 : h0 + h1;
                 }
                 pb[kt] = pk.v;
+                pl[kt] = lo.v;
             }
             psum += __shfl_xor(psum, 16, WAVE);
             psum += __shfl_xor(psum, 32, WAVE);
@@ -738,6 +749,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
                 for (int kt = 0; kt < 4; ++kt) {
                     const s16x4 a = *reinterpret_cast<const s16x4*>(vrow + kt * 16);
                     st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb[kt], st.o[dt], 0, 0, 0);
+                    if (exact) st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl[kt], st.o[dt], 0, 0, 0);
                 }
             }
         }
@@ -783,7 +795,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     bf16_t* __restrict__ out, const int32_t* __restrict__ rows, int n_rows,
     const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
-    float scale, int window, int heads_per_block, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float scale, int window, int heads_per_block, float* __restrict__ part_o, float* __restrict__ part_ml,
+    int exact) {
     constexpr int D = ND * 16, NK = ND / 2;
     // Rows of K lie their length + 32 bytes apart: the fragment reads (row lane % 16, 16-byte piece lane / 16) then
     // meet no bank conflict at any head size (with 16 bytes of padding each read takes 8 cycles instead of 4; counted
@@ -1003,9 +1016,10 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
             // sc[h][s16][i] = score of key kb + 16 s16 + 4 g + i for query (h, lane%16), unscaled. The
             // running maximum is kept unscaled too: a weight is one fused multiply-add and one exp2,
             // exp2((score - max) * scale * log2 e). The vector ALUs are what this kernel is bound by.
-            Frag8 pb[HALVES][2];
+            Frag8 pb[HALVES][2], pl[HALVES][2];
 #pragma unroll
             for (int h = 0; h < HALVES; ++h) {
+                pl[h][0].u = pl[h][1].u = make_uint4(0u, 0u, 0u, 0u);
                 float mx = -INFINITY;
                 if (full) {                               // most tiles: nothing to mask (the same for the whole wave)
 #pragma unroll
@@ -1028,20 +1042,28 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
                 const float m_sub = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;   // exp2(-inf - 0) = 0: masked keys
 #pragma unroll
                 for (int s16 = 0; s16 < 4; ++s16) {
-                    uint32_t pk[2];
+                    uint32_t pk[2], lk[2] = {0u, 0u};
 #pragma unroll
                     for (int i = 0; i < 4; i += 2) {
                         const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[h][s16][i], scale_log2, -m_sub));
                         const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[h][s16][i + 1], scale_log2, -m_sub));
                         pk[i >> 1] = f32x2_to_bf16x2(p0, p1);
+                        // `exact`: what the rounding took off a weight goes through second products (sum and values)
+                        if (exact)
+                            lk[i >> 1] = f32x2_to_bf16x2(p0 - __uint_as_float(pk[i >> 1] << 16),
+                                                         p1 - __uint_as_float(pk[i >> 1] & 0xffff0000u));
                     }
                     // K-slots 4 t + i of group G, s16 = 2 G + t
                     if (s16 & 1) {
                         pb[h][s16 >> 1].u.z = pk[0];
                         pb[h][s16 >> 1].u.w = pk[1];
+                        pl[h][s16 >> 1].u.z = lk[0];
+                        pl[h][s16 >> 1].u.w = lk[1];
                     } else {
                         pb[h][s16 >> 1].u.x = pk[0];
                         pb[h][s16 >> 1].u.y = pk[1];
+                        pl[h][s16 >> 1].u.x = lk[0];
+                        pl[h][s16 >> 1].u.y = lk[1];
                     }
                 }
                 // the old sums shrink by exp2((old max - new max) * scale): by 1, and nothing to do, for
@@ -1056,6 +1078,11 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
 #pragma unroll
                 for (int G = 0; G < 2; ++G)
                     l_acc[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[h][G].v, l_acc[h], 0, 0, 0);
+                if (exact) {
+#pragma unroll
+                    for (int G = 0; G < 2; ++G)
+                        l_acc[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pl[h][G].v, l_acc[h], 0, 0, 0);
+                }
             }
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) {
@@ -1067,6 +1094,11 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
 #pragma unroll
                     for (int h = 0; h < HALVES; ++h)
                         o[h][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pb[h][G].v, o[h][dt], 0, 0, 0);
+                    if (exact) {
+#pragma unroll
+                        for (int h = 0; h < HALVES; ++h)
+                            o[h][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl[h][G].v, o[h][dt], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -1225,7 +1257,7 @@ static int attention_decode_launch(const void* q, const void* k_cache, const voi
                                    const int32_t* seg_start, const int32_t* positions,
                                    const int32_t* block_table, int table_stride, int page_size,
                                    int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
-                                   int n_splits, hipStream_t s, const FromQkv* from_qkv = nullptr) {
+                                   int n_splits, hipStream_t s, const FromQkv* from_qkv = nullptr, int exact = 0) {
     const int G = heads / kv_heads;
     // the merge moves four elements of a head in one access
     if (n_splits > 1 && (((uintptr_t)part_o & 15) || ((uintptr_t)out & 7))) return IMPARO_BAD_ARGUMENT;
@@ -1234,7 +1266,7 @@ static int attention_decode_launch(const void* q, const void* k_cache, const voi
 #define DECODE_FROM_QKV(ND)                                                                                          \
     k_attn_decode<ND, true><<<grid, MFMA_WAVES * 64, 0, s>>>(                                                        \
         nullptr, (const bf16_t*)k_cache, (const bf16_t*)v_cache, part_o, part_ml, (bf16_t*)out, rows, seg_start,     \
-        positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, n_splits, *from_qkv)
+        positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, n_splits, *from_qkv, 0)
         if (head_dim == 64) DECODE_FROM_QKV(4);
         else if (head_dim == 128) DECODE_FROM_QKV(8);
         else return IMPARO_BAD_ARGUMENT;
@@ -1243,7 +1275,7 @@ static int attention_decode_launch(const void* q, const void* k_cache, const voi
         DISPATCH_ND(head_dim / 16, (k_attn_decode<ND, false><<<grid, MFMA_WAVES * 64, 0, s>>>(
             (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, part_o, part_ml, (bf16_t*)out, rows,
             seg_start, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window,
-            n_splits, FromQkv{})));
+            n_splits, FromQkv{}, exact)));
     }
     if (launch_status()) return IMPARO_LAUNCH_FAILED;
     if (n_splits == 1) return IMPARO_OK;
@@ -1252,12 +1284,12 @@ static int attention_decode_launch(const void* q, const void* k_cache, const voi
     return launch_status();
 }
 
-extern "C" int imparo_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
-                                       float* part_o, float* part_ml, const int32_t* rows, int n_rows,
-                                       const int32_t* seg_start, const int32_t* positions,
-                                       const int32_t* block_table, int table_stride, int page_size,
-                                       int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
-                                       int n_splits, imparo_stream stream) {
+static int attention_decode_entry(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                  float* part_o, float* part_ml, const int32_t* rows, int n_rows,
+                                  const int32_t* seg_start, const int32_t* positions,
+                                  const int32_t* block_table, int table_stride, int page_size,
+                                  int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                                  int n_splits, imparo_stream stream, int exact) {
     const int bad = check_common(q, k_cache, v_cache, out, rows, seg_start, positions, block_table, table_stride,
                                  page_size, heads, kv_heads, head_dim, n_pages, window);
     if (bad) return bad;
@@ -1266,7 +1298,31 @@ extern "C" int imparo_attention_decode(const void* q, const void* k_cache, const
     if (n_rows > 65535) return IMPARO_BAD_ARGUMENT;
     return attention_decode_launch(q, k_cache, v_cache, out, part_o, part_ml, rows, n_rows, seg_start, positions,
                                    block_table, table_stride, page_size, heads, kv_heads, head_dim, n_pages, scale,
-                                   window, n_splits, (hipStream_t)stream);
+                                   window, n_splits, (hipStream_t)stream, nullptr, exact);
+}
+
+extern "C" int imparo_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                       float* part_o, float* part_ml, const int32_t* rows, int n_rows,
+                                       const int32_t* seg_start, const int32_t* positions,
+                                       const int32_t* block_table, int table_stride, int page_size,
+                                       int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                                       int n_splits, imparo_stream stream) {
+    return attention_decode_entry(q, k_cache, v_cache, out, part_o, part_ml, rows, n_rows, seg_start, positions,
+                                  block_table, table_stride, page_size, heads, kv_heads, head_dim, n_pages, scale,
+                                  window, n_splits, stream, 0);
+}
+
+// The same with the softmax weights kept to float32 through the product with the values: what rounding a
+// weight to bfloat16 takes off goes through a second product.
+extern "C" int imparo_attention_decode_exact(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                             float* part_o, float* part_ml, const int32_t* rows, int n_rows,
+                                             const int32_t* seg_start, const int32_t* positions,
+                                             const int32_t* block_table, int table_stride, int page_size,
+                                             int heads, int kv_heads, int head_dim, int n_pages, float scale,
+                                             int window, int n_splits, imparo_stream stream) {
+    return attention_decode_entry(q, k_cache, v_cache, out, part_o, part_ml, rows, n_rows, seg_start, positions,
+                                  block_table, table_stride, page_size, heads, kv_heads, head_dim, n_pages, scale,
+                                  window, n_splits, stream, 1);
 }
 
 // Which head sizes and rotations imparo_attention_decode_qkv takes: 64 or 128, rotated whole or not at all.
@@ -1417,13 +1473,13 @@ extern "C" int imparo_attention_prefill_splits(int n_tiles, int heads, int kv_he
     return (int)std::max<long long>(1, std::min<long long>({8, 1024 / blocks, max_context / 1024}));
 }
 
-extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
-                                        float* part_o, float* part_ml, int n_splits,
-                                        const int32_t* rows, int n_rows, int n_tiles,
-                                        const int32_t* seg_start, const int32_t* seg_len, const int32_t* positions,
-                                        const int32_t* block_table, int table_stride, int page_size,
-                                        int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
-                                        imparo_stream stream) {
+static int attention_prefill_entry(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                   float* part_o, float* part_ml, int n_splits,
+                                   const int32_t* rows, int n_rows, int n_tiles,
+                                   const int32_t* seg_start, const int32_t* seg_len, const int32_t* positions,
+                                   const int32_t* block_table, int table_stride, int page_size,
+                                   int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                                   imparo_stream stream, int exact) {
     const int bad = check_common(q, k_cache, v_cache, out, rows, seg_start, positions, block_table, table_stride,
                                  page_size, heads, kv_heads, head_dim, n_pages, window);
     if (bad) return bad;
@@ -1444,7 +1500,7 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
     k_attn_prefill_x32<ND, HALVES, PAGE_TILE><<<grid32, MFMA_WAVES * 64, 0, s>>>(                                    \
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start,     \
         seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb,      \
-        part_o, part_ml)
+        part_o, part_ml, exact)
 #define PREFILL_X32(ND)                                                                                              \
     if (wide && page_size >= PX_KEYS) PREFILL_X32_GO(ND, 2, true);                                                   \
     else if (wide) PREFILL_X32_GO(ND, 2, false);                                                                     \
@@ -1476,8 +1532,34 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
     dim3 grid(n_tiles, heads);
     DISPATCH_ND(head_dim / 16, (k_attn_prefill<ND><<<grid, MFMA_WAVES * 64, 0, s>>>(
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start,
-        seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window)));
+        seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, exact)));
     return launch_status();
+}
+
+extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                        float* part_o, float* part_ml, int n_splits,
+                                        const int32_t* rows, int n_rows, int n_tiles,
+                                        const int32_t* seg_start, const int32_t* seg_len, const int32_t* positions,
+                                        const int32_t* block_table, int table_stride, int page_size,
+                                        int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                                        imparo_stream stream) {
+    return attention_prefill_entry(q, k_cache, v_cache, out, part_o, part_ml, n_splits, rows, n_rows, n_tiles, seg_start,
+                                   seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, head_dim,
+                                   n_pages, scale, window, stream, 0);
+}
+
+// The same with the softmax weights kept to float32 through the product with the values (see
+// imparo_attention_decode_exact).
+extern "C" int imparo_attention_prefill_exact(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                              float* part_o, float* part_ml, int n_splits,
+                                              const int32_t* rows, int n_rows, int n_tiles,
+                                              const int32_t* seg_start, const int32_t* seg_len,
+                                              const int32_t* positions, const int32_t* block_table, int table_stride,
+                                              int page_size, int heads, int kv_heads, int head_dim, int n_pages,
+                                              float scale, int window, imparo_stream stream) {
+    return attention_prefill_entry(q, k_cache, v_cache, out, part_o, part_ml, n_splits, rows, n_rows, n_tiles, seg_start,
+                                   seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, head_dim,
+                                   n_pages, scale, window, stream, 1);
 }
 
 // Asks the runtime about one kernel of this file, which makes it load the file's code onto the

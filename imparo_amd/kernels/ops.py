@@ -273,15 +273,17 @@ def _check_mfma(q, k_cache, v_cache, out):
 
 
 def attention_decode(q, k_cache, v_cache, out, part_o, part_ml, rows, n_rows: int, seg_start, positions,
-                     block_table, scale: float, window: Optional[int], max_context: int) -> torch.Tensor:
+                     block_table, scale: float, window: Optional[int], max_context: int,
+                     exact: bool = False) -> torch.Tensor:
     """Split-KV attention for rows that bring one token each. `rows` lists
-    them (indices into seg_start); `max_context` bounds every row's position + 1."""
+    them (indices into seg_start); `max_context` bounds every row's position + 1.
+    `exact`: the softmax weights keep float32's precision through the product with the values."""
     n, heads, head_dim, n_pages, kv_heads, page_size = _check_mfma(q, k_cache, v_cache, out)
     split = decode_split()
     n_splits = max(1, (max_context + split - 1) // split)
     if part_o.numel() < n_rows * heads * n_splits * head_dim or part_ml.numel() < n_rows * heads * n_splits * 2:
         raise KernelArgumentError("attention_decode: the scratch for partial results is too small")
-    _check(library().imparo_attention_decode(
+    _check((library().imparo_attention_decode_exact if exact else library().imparo_attention_decode)(
         _dev(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
         _dev(part_o, "partial outputs", torch.float32), _dev(part_ml, "partial sums", torch.float32),
         _dev(rows, "decode rows", torch.int32), n_rows, _dev(seg_start, "seg_start", torch.int32),
@@ -344,7 +346,7 @@ def attention_prefill_splits(n_tiles: int, heads: int, kv_heads: int, head_dim: 
 
 def attention_prefill(q, k_cache, v_cache, out, rows, n_rows: int, n_tiles: int, seg_start, seg_len, positions,
                       block_table, scale: float, window: Optional[int], part_o: Optional[torch.Tensor] = None,
-                      part_ml: Optional[torch.Tensor] = None, n_splits: int = 1) -> torch.Tensor:
+                      part_ml: Optional[torch.Tensor] = None, n_splits: int = 1, exact: bool = False) -> torch.Tensor:
     """Tiled attention for rows that bring a portion of a prompt. `n_tiles` is
     the sum over the listed rows of ceil(seg_len / prefill_tile()). With `n_splits` > 1
     (attention_prefill_splits) each block's keys are walked in that many parts,
@@ -358,7 +360,7 @@ def attention_prefill(q, k_cache, v_cache, out, rows, n_rows: int, n_tiles: int,
         _dev(part_ml, "part_ml", torch.float32)
         if part_o.numel() < n * heads * n_splits * head_dim or part_ml.numel() < n * heads * n_splits * 2:
             raise KernelArgumentError("attention_prefill: the buffers for the parts are too small")
-    _check(library().imparo_attention_prefill(
+    _check((library().imparo_attention_prefill_exact if exact else library().imparo_attention_prefill)(
         _dev(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
         part_o.data_ptr() if n_splits > 1 else None, part_ml.data_ptr() if n_splits > 1 else None, int(n_splits),
         _dev(rows, "prefill rows", torch.int32), n_rows, n_tiles, _dev(seg_start, "seg_start", torch.int32),

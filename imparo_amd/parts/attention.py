@@ -14,9 +14,10 @@ layer's cache looks further back than this layer itself; None: everything),
 `shared_kv` (the layer has no key and value projections: it is run with
 another layer's cache, `LayerCall.cache_of`, and brings queries only),
 `weight_suffix` and `names` (how the checkpoint calls the tensors),
-`exact_weights` (the softmax weights stay float32 through the product with the
-values: the wave kernel instead of the matrix-core kernels, which round them
-to bfloat16)."""
+`exact_weights` (the softmax weights keep float32's precision through the
+product with the values: the matrix-core kernels then send what rounding a
+weight to bfloat16 took off through a second product; the wave kernel, which
+takes every other shape, keeps its weights in float32 anyway)."""
 from __future__ import annotations
 
 from typing import Dict, Optional
@@ -112,7 +113,7 @@ class Attention:
         """Keys and values per position, laid out as this mixer's kernels read
         them: where the matrix-core kernels apply (bfloat16, pages of at least
         16, head sizes up to 128), V is kept transposed inside a page."""
-        self.v_transposed = (self.value_dim == self.head_dim and not self.exact_weights
+        self.v_transposed = (self.value_dim == self.head_dim
                              and ops.mfma_attention_supported(self.engine_dtype, page_size, self.head_dim))
         return kv_spec(self.kv_heads, self.head_dim, self.keep_window, self.v_transposed, self.value_dim)
 
@@ -143,7 +144,7 @@ class Attention:
         inv_freq = self.position.inv_freq
         interleaved = bool(getattr(self.position, "interleaved", False))
         Dv = self.value_dim
-        if (vt and owns_cache and Dv == self.head_dim and ctx.single_rows is not None and ctx.n_single_rows == T and not ctx.n_portion_rows
+        if (vt and owns_cache and not self.exact_weights and ctx.single_rows is not None and ctx.n_single_rows == T and not ctx.n_portion_rows
                 and ops.attention_decode_qkv_pays(T, ctx.max_context)
                 and ops.attention_decode_qkv_takes(self.head_dim, 0 if inv_freq is None else inv_freq.shape[0])):
             # every row brings one token: head norm, rotation and the write of the new key and value ride
@@ -167,7 +168,8 @@ class Attention:
             if ctx.n_single_rows:
                 part_o, part_ml = self._decode_parts(ctx)
                 ops.attention_decode(q, k_cache, v_cache, o, part_o, part_ml, ctx.single_rows, ctx.n_single_rows,
-                                     ctx.seg_start, ctx.positions, table, self.scale, self.window, ctx.max_context)
+                                     ctx.seg_start, ctx.positions, table, self.scale, self.window, ctx.max_context,
+                                     exact=self.exact_weights)
             if ctx.n_portion_rows:
                 # few queries over long contexts: each block's keys in parts, merged by a second launch
                 n_tiles = self._portion_tiles(ctx)
@@ -181,7 +183,7 @@ class Attention:
                     part_ml = ctx.workspace.get("attn_prefill_part_ml", (T * self.heads * parts * 2,), torch.float32)
                 ops.attention_prefill(q, k_cache, v_cache, o, ctx.portion_rows, ctx.n_portion_rows,
                                       n_tiles, ctx.seg_start, ctx.seg_len, ctx.positions, table,
-                                      self.scale, self.window, part_o, part_ml, parts)
+                                      self.scale, self.window, part_o, part_ml, parts, exact=self.exact_weights)
         else:
             ops.attention(q, k_cache, v_cache, o, ctx.positions, ctx.row_of_token, table, self.scale, self.window,
                           v_transposed=vt)

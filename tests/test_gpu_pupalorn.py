@@ -222,6 +222,48 @@ def test_a_far_key_among_hundreds(dtype):
     assert float((got - ref).abs().max()) <= (2e-6 if dtype == torch.float32 else 1e-2) * float(ref.abs().max())
 
 
+@pytest.mark.parametrize("D", [64, 128, 48])
+@pytest.mark.parametrize("n_last", [1, 40])
+def test_matrix_core_attention_keeps_its_weights_exact(D, n_last):
+    """Keys in pairs that score nearly alike and carry opposite values: the result is the small difference of
+    two weights, which their rounding to bfloat16 would drown. The matrix-core kernels' exact form must carry
+    it; their plain form, which rounds the weights, must miss it by far (so the case can fail)."""
+    from imparo_amd.kernels import ops
+    H, G, page, L, window = 4, 2, 64, 448, 300
+    g = torch.Generator().manual_seed(D + n_last)
+    bf = lambda t: t.to(torch.bfloat16).float()
+    q, k, v = bf(torch.randn(L, H, D, generator=g)), bf(torch.randn(L, G, D, generator=g)), bf(torch.randn(L, G, D, generator=g))
+    k[1::2] = k[0::2]
+    k[1::2, :, 0] = bf(k[0::2, :, 0] * (1.0 + 2.0 ** -7))
+    v[1::2] = -v[0::2]
+    scale = 1.0 / math.sqrt(D)
+    ref = plain.windowed_attention(q.double(), k.double(), v.double(), torch.arange(L), scale, window)[L - n_last:].float()
+    n_pages = L // page + 2
+    tables = [list(range(n_pages - 1, n_pages - 1 - (L + page - 1) // page, -1))]
+    ctx = hand_context([(L - n_last, n_last)], page, n_pages, torch.bfloat16, torch.device(DEV), tables=tables)
+    kc = torch.zeros(n_pages, G, page, D)
+    vc = torch.zeros(n_pages, G, D, page)
+    for p_ in range(L):
+        kc[tables[0][p_ // page], :, p_ % page] = k[p_]
+        vc[tables[0][p_ // page], :, :, p_ % page] = v[p_]
+    kc, vc, qd = dev(kc, torch.bfloat16), dev(vc, torch.bfloat16), dev(q[L - n_last:], torch.bfloat16)
+    errs = {}
+    for exact in (True, False):
+        out = torch.zeros(n_last, H * D, dtype=torch.bfloat16, device=DEV)
+        if n_last == 1:
+            splits = (L + ops.decode_split() - 1) // ops.decode_split()
+            part_o = torch.zeros(H * splits * D, device=DEV)
+            part_ml = torch.zeros(H * splits * 2, device=DEV)
+            ops.attention_decode(qd, kc, vc, out, part_o, part_ml, ctx.single_rows, 1, ctx.seg_start, ctx.positions,
+                                 ctx.block_tables[0], scale, window, L, exact=exact)
+        else:
+            ops.attention_prefill(qd, kc, vc, out, ctx.portion_rows, 1, (n_last + 63) // 64, ctx.seg_start, ctx.seg_len,
+                                  ctx.positions, ctx.block_tables[0], scale, window, exact=exact)
+        errs[exact] = float((out.float().cpu() - ref).abs().max()) / float(ref.abs().max())
+    assert errs[True] <= 1e-2, errs
+    assert errs[False] > 2 * errs[True], f"rounded weights do not show in this case: {errs}"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,V,rot,n", [(4, 2, 16, 32, 8, 5), (2, 1, 12, 20, 4, 130), (3, 3, 24, 40, 0, 7), (4, 2, 64, 64, 32, 200),
                                            (2, 2, 32, 16, 32, 100)])
