@@ -442,7 +442,7 @@ int imparo_moe_plan(const int32_t* choice, int n_entries, int n_experts, int til
                     imparo_stream stream);
 // product: out[slot, :n] = epilogue(a[row(slot), :k] . w[expert(slot), :n, :k]); row(slot) is the slot, or with
 // gather_div > 0 entry_of_slot[slot] / gather_div. epilogue 0: none, 1: max(z, 0)^2. bfloat16 operands (k a
-// multiple of 8, out bfloat16 or float32) or float32 throughout (tile_rows 64).
+// multiple of 8, out bfloat16 or float32; tile_rows 16, 64 or 128) or float32 throughout (tile_rows 64).
 int imparo_moe_gemm(const void* a, int a_ld, int gather_div, const int32_t* entry_of_slot, const void* w,
                     void* out, int out_dtype, int dtype, const int32_t* tiles, int max_tiles, int tile_rows,
                     int n, int k, int epilogue, imparo_stream stream);

@@ -150,9 +150,10 @@ extern "C" int imparo_moe_max_tiles(int n_entries, int n_experts, int tile_rows)
 }
 
 // Rows of a product's tile for this many entries over this many experts: the wide tile where an
-// expert's share fills it, the narrow one else (a decode step, many experts).
+// expert's share fills it, the narrow one else (many experts), tiles of 16 for the few entries of a decode step.
 extern "C" int imparo_moe_tile_rows(int n_entries, int n_experts, int dtype) {
     if (dtype != IMPARO_BF16) return 64;
+    if (n_entries <= 128) return 16;          // a decode step: the experts' matrices are streamed once, few rows each
     return (n_experts > 0 && n_entries / n_experts >= 96) ? 128 : 64;
 }
 
@@ -179,11 +180,6 @@ __device__ __forceinline__ float moe_epilogue(float v, int epi) {
     }
     return v;
 }
-
-union MoeFrag {
-    uint4 u;
-    bf16x8 v;
-};
 
 // out[slot, n] = epi(sum_k a[row(slot), k] * w[expert, n, k]) for the slots of one tile. row(slot) is the
 // slot itself, or with gather_div the token of the slot's entry (entry / gather_div). Four waves as 2 x 2,
@@ -215,31 +211,46 @@ __global__ __launch_bounds__(256) void k_moe_gemm_bf16(const bf16_t* __restrict_
     }
 #pragma unroll
     for (int j = 0; j < TN / 32; ++j) pb[j] = Wb + (size_t)min(n0 + (tid >> 3) + 32 * j, N - 1) * K;
-    uint4 ra[TM / 32], rb[TN / 32];
-    const uint4 zero = {0u, 0u, 0u, 0u};
-    auto fetch = [&](int kt) {
-        const int k = kt * BK + kc;
-        const bool in = k < K;
-        const int kk = in ? k : 0;
-#pragma unroll
-        for (int j = 0; j < TM / 32; ++j) {
-            const uint4 v = *reinterpret_cast<const uint4*>(pa[j] + kk);
-            ra[j] = in ? v : zero;
-        }
-#pragma unroll
-        for (int j = 0; j < TN / 32; ++j) {
-            const uint4 v = *reinterpret_cast<const uint4*>(pb[j] + kk);
-            rb[j] = in ? v : zero;
-        }
-    };
-    auto stash = [&](int buf) {
-#pragma unroll
-        for (int j = 0; j < TM / 32; ++j)
-            *reinterpret_cast<uint4*>(&As[buf][((tid >> 3) + 32 * j) * LD + kc]) = ra[j];
-#pragma unroll
-        for (int j = 0; j < TN / 32; ++j)
-            *reinterpret_cast<uint4*>(&Bs[buf][((tid >> 3) + 32 * j) * LD + kc]) = rb[j];
-    };
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    // two sets of registers, each holding one K-step's loads: a step's loads are asked for two steps ahead
+    u32x4 ra0[TM / 32], rb0[TN / 32], ra1[TM / 32], rb1[TN / 32];
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    const int nk = (K + BK - 1) / BK;
+    // the loads of K-step kt into registers; what lies beyond K comes as zeros (K is a multiple of 8, so a
+    // piece of 8 is inside or outside as a whole) from an address inside the row; a step past the last
+    // reads the last again and is never stored
+#define MOE_FETCH(kt, ra, rb)                                                                                       \
+    {                                                                                                               \
+        const int k_ = min((kt), nk - 1) * BK + kc;                                                                 \
+        const bool in_ = k_ < K;                                                                                    \
+        const int kk_ = in_ ? k_ : 0;                                                                               \
+        _Pragma("unroll") for (int j = 0; j < TM / 32; ++j) {                                                       \
+            const u32x4 v_ = *reinterpret_cast<const u32x4*>(pa[j] + kk_);                                          \
+            ra[j] = in_ ? v_ : zero;                                                                                \
+        }                                                                                                           \
+        _Pragma("unroll") for (int j = 0; j < TN / 32; ++j) {                                                       \
+            const u32x4 v_ = *reinterpret_cast<const u32x4*>(pb[j] + kk_);                                          \
+            rb[j] = in_ ? v_ : zero;                                                                                \
+        }                                                                                                           \
+    }
+#define MOE_STASH(buf_, ra, rb)                                                                                     \
+    {                                                                                                               \
+        _Pragma("unroll") for (int j = 0; j < TM / 32; ++j)                                                         \
+            *reinterpret_cast<u32x4*>(&As[buf_][((tid >> 3) + 32 * j) * LD + kc]) = ra[j];                          \
+        _Pragma("unroll") for (int j = 0; j < TN / 32; ++j)                                                         \
+            *reinterpret_cast<u32x4*>(&Bs[buf_][((tid >> 3) + 32 * j) * LD + kc]) = rb[j];                          \
+    }
+#define MOE_MULTIPLY(buf_)                                                                                          \
+    _Pragma("unroll") for (int ks = 0; ks < BK / 16; ++ks) {                                                        \
+        bf16x8 fa[WM], fb[WN];                                                                                      \
+        _Pragma("unroll") for (int i = 0; i < WM; ++i)                                                              \
+            fa[i] = *reinterpret_cast<const bf16x8*>(&As[buf_][a_base + i * 32 * LD + ks * 16]);                    \
+        _Pragma("unroll") for (int j = 0; j < WN; ++j)                                                              \
+            fb[j] = *reinterpret_cast<const bf16x8*>(&Bs[buf_][b_base + j * 32 * LD + ks * 16]);                    \
+        _Pragma("unroll") for (int i = 0; i < WM; ++i)                                                              \
+            _Pragma("unroll") for (int j = 0; j < WN; ++j)                                                          \
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);              \
+    }
     f32x16 acc[WM][WN];
 #pragma unroll
     for (int i = 0; i < WM; ++i)
@@ -249,31 +260,28 @@ __global__ __launch_bounds__(256) void k_moe_gemm_bf16(const bf16_t* __restrict_
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     const int a_base = (wm * 32 * WM + (lane & 31)) * LD + (lane >> 5) * 8;
     const int b_base = (wn * 32 * WN + (lane & 31)) * LD + (lane >> 5) * 8;
-    const int nk = (K + BK - 1) / BK;
-    fetch(0);
-    stash(0);
+    MOE_FETCH(0, ra0, rb0);
+    MOE_FETCH(1, ra1, rb1);
+    MOE_STASH(0, ra0, rb0);
+    MOE_FETCH(2, ra0, rb0);
     __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) fetch(kt + 1);
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            MoeFrag fa[WM], fb[WN];
-#pragma unroll
-            for (int i = 0; i < WM; ++i)
-                fa[i].u = *reinterpret_cast<const uint4*>(&As[buf][a_base + i * 32 * LD + ks * 16]);
-#pragma unroll
-            for (int j = 0; j < WN; ++j)
-                fb[j].u = *reinterpret_cast<const uint4*>(&Bs[buf][b_base + j * 32 * LD + ks * 16]);
-#pragma unroll
-            for (int i = 0; i < WM; ++i)
-#pragma unroll
-                for (int j = 0; j < WN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i].v, fb[j].v, acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nk) stash(buf ^ 1);
+    // step kt is multiplied out of stage kt % 2 while step kt + 1 goes from its registers into the other
+    // stage and those registers take the loads of step kt + 3
+    for (int kt = 0; kt < nk; kt += 2) {
+        MOE_MULTIPLY(0);
+        if (kt + 1 < nk) MOE_STASH(1, ra1, rb1);
+        MOE_FETCH(kt + 3, ra1, rb1);
         __syncthreads();
+        if (kt + 1 < nk) {
+            MOE_MULTIPLY(1);
+            if (kt + 2 < nk) MOE_STASH(0, ra0, rb0);
+            MOE_FETCH(kt + 4, ra0, rb0);
+            __syncthreads();
+        }
     }
+#undef MOE_FETCH
+#undef MOE_STASH
+#undef MOE_MULTIPLY
     // a lane holds column lane % 32 of a 32 x 32 product, rows 8 (r / 4) + 4 (lane / 32) + r % 4
 #pragma unroll
     for (int i = 0; i < WM; ++i)
@@ -286,6 +294,76 @@ __global__ __launch_bounds__(256) void k_moe_gemm_bf16(const bf16_t* __restrict_
                 if (m < rows && n < N) store_f32<TOut>(out, (size_t)(row0 + m) * N + n, moe_epilogue(acc[i][j][r], epi));
             }
         }
+}
+
+// Few rows an expert (a decode step): a block takes 16 outputs of one expert and up to 16 slots. The expert's
+// 16 weight rows are the M side of 16x16x32 products and go from memory straight into the operand registers,
+// K cut over the block's four waves and, inside a wave, walked in runs of 64 with four runs' loads in flight
+// (a lane takes 16 consecutive k of its row, so that four lanes read a row's 128 bytes side by side; the
+// slots' rows are read with the same k order, which is all a dot product asks for). The waves' partial sums
+// meet in LDS and are added in wave order.
+template <typename TOut>
+__global__ __launch_bounds__(256) void k_moe_gemm_rows16(const bf16_t* __restrict__ A, int a_ld, int gather_div,
+                                                         const int32_t* __restrict__ entry_of_slot,
+                                                         const bf16_t* __restrict__ W, TOut* __restrict__ out,
+                                                         const int32_t* __restrict__ tiles, int N, int K, int epi) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    __shared__ f32x4 part[4][WAVE];
+    const int expert = tiles[3 * blockIdx.x];
+    if (expert < 0) return;
+    const int row0 = tiles[3 * blockIdx.x + 1], rows = tiles[3 * blockIdx.x + 2];
+    const int n0 = blockIdx.y * 16;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const bf16_t* wrow = W + ((size_t)expert * N + min(n0 + c, N - 1)) * K;
+    const int slot = row0 + min(c, rows - 1);
+    const bf16_t* arow = A + (size_t)(gather_div ? entry_of_slot[slot] / gather_div : slot) * a_ld;
+    // this wave's part of K, in whole runs of 64
+    const int runs = (K + 63) / 64;
+    const int per_wave = (runs + 3) / 4;
+    const int run_lo = wave * per_wave, run_hi = min(runs, run_lo + per_wave);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    for (int r0 = run_lo; r0 < run_hi; r0 += 4) {
+        u32x4 w[4][2], a[4][2];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int k = min(r0 + u, run_hi - 1) * 64 + g * 16 + h * 8;
+                const bool in = k < K && r0 + u < run_hi;
+                const int kk = k < K ? k : 0;
+                const u32x4 wv = *reinterpret_cast<const u32x4*>(wrow + kk);
+                const u32x4 av = *reinterpret_cast<const u32x4*>(arow + kk);
+                w[u][h] = in ? wv : zero;
+                a[u][h] = in ? av : zero;
+            }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w[u][h]),
+                                                              __builtin_bit_cast(bf16x8, a[u][h]), acc, 0, 0, 0);
+    }
+    part[wave][lane] = acc;
+    __syncthreads();
+    if (wave != 0) return;
+    f32x4 total = part[0][lane];
+#pragma unroll
+    for (int w2 = 1; w2 < 4; ++w2) {
+        const f32x4 p = part[w2][lane];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) total[i] += p[i];
+    }
+    // a lane holds slot c, outputs n0 + 4 g + i
+    if (c < rows) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + 4 * g + i;
+            if (n < N) store_f32<TOut>(out, (size_t)(row0 + c) * N + n, moe_epilogue(total[i], epi));
+        }
+    }
 }
 
 // The same in float32: a tile of 64 slots by 64 outputs, K in steps of 16 through LDS, every output
@@ -367,7 +445,17 @@ extern "C" int imparo_moe_gemm(const void* a, int a_ld, int gather_div, const in
 #define MOE_LAUNCH(WM, WN, TO)                                                                                       \
     k_moe_gemm_bf16<WM, WN, TO><<<dim3(max_tiles, (n + 64 * WN - 1) / (64 * WN)), 256, 0, s>>>(                      \
         (const bf16_t*)a, a_ld, gather_div, entry_of_slot, (const bf16_t*)w, (TO*)out, tiles, n, k, epilogue)
-    if (tile_rows == 128) {
+    if (tile_rows == 16) {
+        const dim3 grid16(max_tiles, (n + 15) / 16);
+        if (out_dtype == IMPARO_BF16)
+            k_moe_gemm_rows16<bf16_t><<<grid16, 256, 0, s>>>((const bf16_t*)a, a_ld, gather_div, entry_of_slot,
+                                                             (const bf16_t*)w, (bf16_t*)out, tiles, n, k, epilogue);
+        else if (out_dtype == IMPARO_F32)
+            k_moe_gemm_rows16<float><<<grid16, 256, 0, s>>>((const bf16_t*)a, a_ld, gather_div, entry_of_slot,
+                                                            (const bf16_t*)w, (float*)out, tiles, n, k, epilogue);
+        else
+            return IMPARO_BAD_ARGUMENT;
+    } else if (tile_rows == 128) {
         if (out_dtype == IMPARO_BF16) MOE_LAUNCH(2, 2, bf16_t);
         else if (out_dtype == IMPARO_F32) MOE_LAUNCH(2, 2, float);
         else return IMPARO_BAD_ARGUMENT;
@@ -436,38 +524,55 @@ extern "C" int imparo_moe_combine(const float* y, const void* h, int h_dtype, co
 // ---------------------------------------------------------------- a norm on what a sublayer returns
 // x[row] += d / sqrt(mean(d^2) + eps_post) * w_post, d = the sum of the delta's slices in order; then,
 // with w_next, out[row] = x[row] / sqrt(mean(x[row]^2) + eps_next) * w_next. One block a row, the row in
-// LDS between the passes, every sum in float32 and in an order that the width alone decides. With `rows`
+// registers between the passes, every sum in float32 and in an order that the width alone decides. With `rows`
 // only those rows are taken and the stream is left as it is (the rows whose logits are wanted).
-template <typename TOut>
+// PER: values of the row a thread keeps in registers (the block's threads x PER cover the width); every
+// load of the row (the delta's slices, the stream, both weights) is asked for before any is used.
+template <typename TOut, int PER>
 __global__ __launch_bounds__(256) void k_post_norm_add(float* __restrict__ x, const float* __restrict__ delta,
                                                        int n_delta, size_t delta_stride,
                                                        const int32_t* __restrict__ rows,
                                                        const float* __restrict__ w_post, float eps_post,
                                                        const float* __restrict__ w_next, float eps_next,
                                                        TOut* __restrict__ out, int width, int write_back) {
-    extern __shared__ float row[];
     __shared__ float scratch[16];
     const int i_out = blockIdx.x;
     const size_t src = (size_t)(rows ? rows[i_out] : i_out) * width;
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        float d = delta[src + i];
-        for (int s = 1; s < n_delta; ++s) d += delta[(size_t)s * delta_stride + src + i];
-        row[i] = d;
-        ss = fmaf(d, d, ss);
+    float d[PER], xv[PER], wp[PER], wn[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = threadIdx.x + j * 256;
+        const int ii = min(i, width - 1);
+        d[j] = delta[src + ii];
+        xv[j] = x[src + ii];
+        wp[j] = w_post[ii];
+        wn[j] = w_next ? w_next[ii] : 0.f;
     }
+    for (int s = 1; s < n_delta; ++s)
+#pragma unroll
+        for (int j = 0; j < PER; ++j) d[j] += delta[(size_t)s * delta_stride + src + min((int)threadIdx.x + j * 256, width - 1)];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+        if (threadIdx.x + j * 256 < width) ss = fmaf(d[j], d[j], ss);
     const float r1 = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps_post);
     ss = 0.f;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        const float v = x[src + i] + row[i] * r1 * w_post[i];
-        row[i] = v;
-        if (write_back) x[src + i] = v;
-        ss = fmaf(v, v, ss);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = threadIdx.x + j * 256;
+        xv[j] = xv[j] + d[j] * r1 * wp[j];
+        if (i < width) {
+            if (write_back) x[src + i] = xv[j];
+            ss = fmaf(xv[j], xv[j], ss);
+        }
     }
     if (!w_next) return;
     const float r2 = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps_next);
-    for (int i = threadIdx.x; i < width; i += blockDim.x)
-        store_f32<TOut>(out, (size_t)i_out * width + i, row[i] * r2 * w_next[i]);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = threadIdx.x + j * 256;
+        if (i < width) store_f32<TOut>(out, (size_t)i_out * width + i, xv[j] * r2 * wn[j]);
+    }
 }
 
 extern "C" int imparo_post_norm_add(float* x, const float* delta, int n_delta, int n_rows_x, const int32_t* rows,
@@ -481,15 +586,24 @@ extern "C" int imparo_post_norm_add(float* x, const float* delta, int n_delta, i
     hipStream_t s = (hipStream_t)stream;
     const size_t stride = (size_t)n_rows_x * width;
     const int write_back = rows ? 0 : 1;
-    const size_t lds = (size_t)width * sizeof(float);
-    if (!w_next || out_dtype == IMPARO_F32)
-        k_post_norm_add<float><<<n_out, 256, lds, s>>>(x, delta, n_delta, stride, rows, w_post, eps_post, w_next,
-                                                       eps_next, (float*)out, width, write_back);
-    else if (out_dtype == IMPARO_BF16)
-        k_post_norm_add<bf16_t><<<n_out, 256, lds, s>>>(x, delta, n_delta, stride, rows, w_post, eps_post, w_next,
-                                                        eps_next, (bf16_t*)out, width, write_back);
-    else
-        return IMPARO_BAD_ARGUMENT;
+    const bool to_bf16 = w_next && out_dtype == IMPARO_BF16;
+    if (w_next && out_dtype != IMPARO_BF16 && out_dtype != IMPARO_F32) return IMPARO_BAD_ARGUMENT;
+#define POST_NORM(PER)                                                                                              \
+    if (to_bf16)                                                                                                    \
+        k_post_norm_add<bf16_t, PER><<<n_out, 256, 0, s>>>(x, delta, n_delta, stride, rows, w_post, eps_post,       \
+                                                           w_next, eps_next, (bf16_t*)out, width, write_back);      \
+    else                                                                                                            \
+        k_post_norm_add<float, PER><<<n_out, 256, 0, s>>>(x, delta, n_delta, stride, rows, w_post, eps_post,        \
+                                                          w_next, eps_next, (float*)out, width, write_back)
+    const int per = (width + 255) / 256;
+    if (per <= 1) { POST_NORM(1); }
+    else if (per <= 2) { POST_NORM(2); }
+    else if (per <= 4) { POST_NORM(4); }
+    else if (per <= 8) { POST_NORM(8); }
+    else if (per <= 16) { POST_NORM(16); }
+    else if (per <= 32) { POST_NORM(32); }
+    else { POST_NORM(64); }
+#undef POST_NORM
     return launch_status();
 }
 
