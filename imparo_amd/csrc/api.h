@@ -451,12 +451,27 @@ int imparo_moe_combine(const float* y, const void* h, int h_dtype, const int32_t
                        const float* weight, const int32_t* slot_of_entry, float* out, int n_tokens,
                        int width, int top, int n_experts, imparo_stream stream);
 
+// route and plan in one launch, for at most imparo_moe_route_plan_tokens() tokens (a decode step)
+int imparo_moe_route_plan_tokens(void);
+int imparo_moe_route_plan(const float* logits, const float* correction, int32_t* choice, float* weight,
+                          int n_tokens, int n_router, int top, int n_experts, int tile_rows,
+                          int32_t* slot_of_entry, int32_t* entry_of_slot, int32_t* tiles, int max_tiles,
+                          imparo_stream stream);
+
 // A norm on what a sublayer returns, its add into the stream, and the next norm, in one launch:
 // x[r] += rms_norm(sum of delta's slices [n_delta, n_rows_x, width])[r] * w_post; with w_next,
 // out[i] = rms_norm(x[r]) * w_next. r = rows[i] (then x is left as it is), or i.
 int imparo_post_norm_add(float* x, const float* delta, int n_delta, int n_rows_x, const int32_t* rows,
                          const float* w_post, float eps_post, const float* w_next, float eps_next,
                          void* out, int out_dtype, int n_out, int width, imparo_stream stream);
+
+// imparo_post_norm_add with the delta made in the launch from a routed feed-forward's rows: what
+// imparo_moe_combine would have written, added up in the same order.
+int imparo_post_norm_add_moe(float* x, const float* y, const void* h, int h_dtype, const int32_t* choice,
+                             const float* weight, const int32_t* slot_of_entry, int top, int n_experts,
+                             int n_rows_x, const int32_t* rows, const float* w_post, float eps_post,
+                             const float* w_next, float eps_next, void* out, int out_dtype, int n_out,
+                             int width, imparo_stream stream);
 
 #ifdef __cplusplus
 }

@@ -21,13 +21,13 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define MOE_MAX_EXPERTS 1024        // real experts the plan kernel keeps counters for
 #define MOE_MAX_TOP 16
 
+extern "C" int imparo_moe_max_tiles(int n_entries, int n_experts, int tile_rows);
+
 // ---------------------------------------------------------------- route
-__global__ void k_moe_route(const float* __restrict__ logits, const float* __restrict__ correction,
-                            int32_t* __restrict__ choice, float* __restrict__ weight, int n_tokens, int n_router,
-                            int top) {
+__device__ __forceinline__ void moe_route_token(const float* __restrict__ logits, const float* __restrict__ correction,
+                                                int32_t* __restrict__ choice, float* __restrict__ weight, int t,
+                                                int n_router, int top) {
     const int lane = threadIdx.x & (WAVE - 1);
-    const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-    if (t >= n_tokens) return;
     constexpr int PER = MOE_MAX_ROUTER / WAVE;
     float z[PER], pick[PER];
     float m = -INFINITY;
@@ -79,6 +79,13 @@ __global__ void k_moe_route(const float* __restrict__ logits, const float* __res
     }
 }
 
+__global__ void k_moe_route(const float* __restrict__ logits, const float* __restrict__ correction,
+                            int32_t* __restrict__ choice, float* __restrict__ weight, int n_tokens, int n_router,
+                            int top) {
+    const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (t < n_tokens) moe_route_token(logits, correction, choice, weight, t, n_router, top);
+}
+
 extern "C" int imparo_moe_route(const float* logits, const float* correction, int32_t* choice, float* weight,
                                 int n_tokens, int n_router, int top, imparo_stream stream) {
     if (!logits || !choice || !weight || n_tokens < 0) return IMPARO_BAD_ARGUMENT;
@@ -92,11 +99,17 @@ extern "C" int imparo_moe_route(const float* logits, const float* correction, in
 
 // ---------------------------------------------------------------- plan
 // tiles[3 i ..]: expert, first slot, rows of tile i; expert -1 where the list has ended.
-__global__ __launch_bounds__(1024) void k_moe_plan(const int32_t* __restrict__ choice, int n_entries, int n_experts,
-                                                   int tile_rows, int32_t* __restrict__ slot_of_entry,
-                                                   int32_t* __restrict__ entry_of_slot, int32_t* __restrict__ tiles,
-                                                   int max_tiles) {
-    __shared__ int count[MOE_MAX_EXPERTS], first[MOE_MAX_EXPERTS], first_tile[MOE_MAX_EXPERTS + 1];
+struct MoePlanShared {
+    int count[MOE_MAX_EXPERTS], first[MOE_MAX_EXPERTS], first_tile[MOE_MAX_EXPERTS + 1];
+};
+
+__device__ __forceinline__ void moe_plan_block(MoePlanShared& sh, const int32_t* __restrict__ choice, int n_entries,
+                                               int n_experts, int tile_rows, int32_t* __restrict__ slot_of_entry,
+                                               int32_t* __restrict__ entry_of_slot, int32_t* __restrict__ tiles,
+                                               int max_tiles) {
+    int* count = sh.count;
+    int* first = sh.first;
+    int* first_tile = sh.first_tile;
     const int tid = threadIdx.x;
     for (int e = tid; e < n_experts; e += blockDim.x) count[e] = 0;
     __syncthreads();
@@ -142,6 +155,51 @@ __global__ __launch_bounds__(1024) void k_moe_plan(const int32_t* __restrict__ c
         }
         slot_of_entry[i] = slot;
     }
+}
+
+__global__ __launch_bounds__(1024) void k_moe_plan(const int32_t* __restrict__ choice, int n_entries, int n_experts,
+                                                   int tile_rows, int32_t* __restrict__ slot_of_entry,
+                                                   int32_t* __restrict__ entry_of_slot, int32_t* __restrict__ tiles,
+                                                   int max_tiles) {
+    __shared__ MoePlanShared sh;
+    moe_plan_block(sh, choice, n_entries, n_experts, tile_rows, slot_of_entry, entry_of_slot, tiles, max_tiles);
+}
+
+// Route and plan in one launch, for the few tokens of a decode step: the block's waves route the tokens in
+// turn, then the block plans what they chose.
+#define MOE_ROUTE_PLAN_TOKENS 64
+__global__ __launch_bounds__(1024) void k_moe_route_plan(const float* __restrict__ logits,
+                                                         const float* __restrict__ correction,
+                                                         int32_t* __restrict__ choice, float* __restrict__ weight,
+                                                         int n_tokens, int n_router, int top, int n_experts,
+                                                         int tile_rows, int32_t* __restrict__ slot_of_entry,
+                                                         int32_t* __restrict__ entry_of_slot,
+                                                         int32_t* __restrict__ tiles, int max_tiles) {
+    __shared__ MoePlanShared sh;
+    for (int t = threadIdx.x / WAVE; t < n_tokens; t += blockDim.x / WAVE)
+        moe_route_token(logits, correction, choice, weight, t, n_router, top);
+    __threadfence_block();
+    __syncthreads();
+    moe_plan_block(sh, choice, n_tokens * top, n_experts, tile_rows, slot_of_entry, entry_of_slot, tiles, max_tiles);
+}
+
+extern "C" int imparo_moe_route_plan_tokens() { return MOE_ROUTE_PLAN_TOKENS; }
+
+extern "C" int imparo_moe_route_plan(const float* logits, const float* correction, int32_t* choice, float* weight,
+                                     int n_tokens, int n_router, int top, int n_experts, int tile_rows,
+                                     int32_t* slot_of_entry, int32_t* entry_of_slot, int32_t* tiles, int max_tiles,
+                                     imparo_stream stream) {
+    if (!logits || !choice || !weight || !slot_of_entry || !entry_of_slot || !tiles) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens < 0 || n_tokens > MOE_ROUTE_PLAN_TOKENS) return IMPARO_BAD_ARGUMENT;
+    if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > n_router || top > MOE_MAX_TOP)
+        return IMPARO_BAD_ARGUMENT;
+    if (n_experts < 0 || n_experts > MOE_MAX_EXPERTS || tile_rows < 1) return IMPARO_BAD_ARGUMENT;
+    if (max_tiles < imparo_moe_max_tiles(n_tokens * top, n_experts, tile_rows)) return IMPARO_SCRATCH_TOO_SMALL;
+    if (n_tokens == 0) return IMPARO_OK;
+    k_moe_route_plan<<<1, 1024, 0, (hipStream_t)stream>>>(logits, correction, choice, weight, n_tokens, n_router, top,
+                                                          n_experts, tile_rows, slot_of_entry, entry_of_slot, tiles,
+                                                          max_tiles);
+    return launch_status();
 }
 
 extern "C" int imparo_moe_max_tiles(int n_entries, int n_experts, int tile_rows) {
@@ -528,9 +586,21 @@ extern "C" int imparo_moe_combine(const float* y, const void* h, int h_dtype, co
 // only those rows are taken and the stream is left as it is (the rows whose logits are wanted).
 // PER: values of the row a thread keeps in registers (the block's threads x PER cover the width); every
 // load of the row (the delta's slices, the stream, both weights) is asked for before any is used.
+// What a routed feed-forward leaves for this launch to combine instead of a finished delta: the experts'
+// rows y [slots, width], the feed-forward's input h (for experts that pass it through), and per token its
+// choice, weights and slots. delta[t] = sum_j weight[t, j] * (y[slot] or h[t]), j in the order of the choice.
+struct MoeRows {
+    const float* y;
+    const void* h;
+    const int32_t* choice;
+    const float* weight;
+    const int32_t* slot_of_entry;
+    int h_is_bf16, top, n_experts;
+};
+
 template <typename TOut, int PER>
 __global__ __launch_bounds__(256) void k_post_norm_add(float* __restrict__ x, const float* __restrict__ delta,
-                                                       int n_delta, size_t delta_stride,
+                                                       int n_delta, size_t delta_stride, MoeRows moe,
                                                        const int32_t* __restrict__ rows,
                                                        const float* __restrict__ w_post, float eps_post,
                                                        const float* __restrict__ w_next, float eps_next,
@@ -539,16 +609,41 @@ __global__ __launch_bounds__(256) void k_post_norm_add(float* __restrict__ x, co
     const int i_out = blockIdx.x;
     const size_t src = (size_t)(rows ? rows[i_out] : i_out) * width;
     float d[PER], xv[PER], wp[PER], wn[PER];
+    if (moe.y) {
+        __shared__ int slot[MOE_MAX_TOP];
+        __shared__ float wt[MOE_MAX_TOP];
+        const size_t t = src / width;
+        if ((int)threadIdx.x < moe.top) {
+            const int e = moe.choice[t * moe.top + threadIdx.x];
+            slot[threadIdx.x] = e < moe.n_experts ? moe.slot_of_entry[t * moe.top + threadIdx.x] : -1;
+            wt[threadIdx.x] = moe.weight[t * moe.top + threadIdx.x];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < PER; ++j) d[j] = 0.f;
+        for (int k = 0; k < moe.top; ++k) {
+            const int sl = slot[k];
+            const float w = wt[k];
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                const int ii = min((int)threadIdx.x + j * 256, width - 1);
+                const float v = sl >= 0 ? moe.y[(size_t)sl * width + ii]
+                                        : (moe.h_is_bf16 ? load_f32<bf16_t>((const bf16_t*)moe.h, src + ii)
+                                                         : load_f32<float>((const float*)moe.h, src + ii));
+                d[j] = fmaf(w, v, d[j]);
+            }
+        }
+    }
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int i = threadIdx.x + j * 256;
         const int ii = min(i, width - 1);
-        d[j] = delta[src + ii];
+        if (!moe.y) d[j] = delta[src + ii];
         xv[j] = x[src + ii];
         wp[j] = w_post[ii];
         wn[j] = w_next ? w_next[ii] : 0.f;
     }
-    for (int s = 1; s < n_delta; ++s)
+    for (int s = 1; s < n_delta && !moe.y; ++s)
 #pragma unroll
         for (int j = 0; j < PER; ++j) d[j] += delta[(size_t)s * delta_stride + src + min((int)threadIdx.x + j * 256, width - 1)];
     float ss = 0.f;
@@ -575,10 +670,10 @@ __global__ __launch_bounds__(256) void k_post_norm_add(float* __restrict__ x, co
     }
 }
 
-extern "C" int imparo_post_norm_add(float* x, const float* delta, int n_delta, int n_rows_x, const int32_t* rows,
-                                    const float* w_post, float eps_post, const float* w_next, float eps_next,
-                                    void* out, int out_dtype, int n_out, int width, imparo_stream stream) {
-    if (!x || !delta || !w_post || n_delta < 1 || n_rows_x < 0 || n_out < 0 || width < 1 || width > 16384)
+static int post_norm_add_launch(float* x, const float* delta, int n_delta, MoeRows moe, int n_rows_x,
+                                const int32_t* rows, const float* w_post, float eps_post, const float* w_next,
+                                float eps_next, void* out, int out_dtype, int n_out, int width, imparo_stream stream) {
+    if (!x || (!delta && !moe.y) || !w_post || n_delta < 1 || n_rows_x < 0 || n_out < 0 || width < 1 || width > 16384)
         return IMPARO_BAD_ARGUMENT;
     if (w_next && !out) return IMPARO_BAD_ARGUMENT;
     if (!rows && n_out != n_rows_x) return IMPARO_BAD_ARGUMENT;
@@ -590,10 +685,10 @@ extern "C" int imparo_post_norm_add(float* x, const float* delta, int n_delta, i
     if (w_next && out_dtype != IMPARO_BF16 && out_dtype != IMPARO_F32) return IMPARO_BAD_ARGUMENT;
 #define POST_NORM(PER)                                                                                              \
     if (to_bf16)                                                                                                    \
-        k_post_norm_add<bf16_t, PER><<<n_out, 256, 0, s>>>(x, delta, n_delta, stride, rows, w_post, eps_post,       \
+        k_post_norm_add<bf16_t, PER><<<n_out, 256, 0, s>>>(x, delta, n_delta, stride, moe, rows, w_post, eps_post,  \
                                                            w_next, eps_next, (bf16_t*)out, width, write_back);      \
     else                                                                                                            \
-        k_post_norm_add<float, PER><<<n_out, 256, 0, s>>>(x, delta, n_delta, stride, rows, w_post, eps_post,        \
+        k_post_norm_add<float, PER><<<n_out, 256, 0, s>>>(x, delta, n_delta, stride, moe, rows, w_post, eps_post,   \
                                                           w_next, eps_next, (float*)out, width, write_back)
     const int per = (width + 255) / 256;
     if (per <= 1) { POST_NORM(1); }
@@ -605,6 +700,27 @@ extern "C" int imparo_post_norm_add(float* x, const float* delta, int n_delta, i
     else { POST_NORM(64); }
 #undef POST_NORM
     return launch_status();
+}
+
+extern "C" int imparo_post_norm_add(float* x, const float* delta, int n_delta, int n_rows_x, const int32_t* rows,
+                                    const float* w_post, float eps_post, const float* w_next, float eps_next,
+                                    void* out, int out_dtype, int n_out, int width, imparo_stream stream) {
+    return post_norm_add_launch(x, delta, n_delta, MoeRows{}, n_rows_x, rows, w_post, eps_post, w_next, eps_next, out,
+                                out_dtype, n_out, width, stream);
+}
+
+// The same with the delta made in the launch from a routed feed-forward's rows (imparo_moe_combine's sum).
+extern "C" int imparo_post_norm_add_moe(float* x, const float* y, const void* h, int h_dtype, const int32_t* choice,
+                                        const float* weight, const int32_t* slot_of_entry, int top, int n_experts,
+                                        int n_rows_x, const int32_t* rows, const float* w_post, float eps_post,
+                                        const float* w_next, float eps_next, void* out, int out_dtype, int n_out,
+                                        int width, imparo_stream stream) {
+    if (!y || !h || !choice || !weight || !slot_of_entry || top < 1 || top > MOE_MAX_TOP || n_experts < 0)
+        return IMPARO_BAD_ARGUMENT;
+    if (h_dtype != IMPARO_F32 && h_dtype != IMPARO_BF16) return IMPARO_BAD_ARGUMENT;
+    const MoeRows moe{y, h, choice, weight, slot_of_entry, h_dtype == IMPARO_BF16, top, n_experts};
+    return post_norm_add_launch(x, nullptr, 1, moe, n_rows_x, rows, w_post, eps_post, w_next, eps_next, out, out_dtype,
+                                n_out, width, stream);
 }
 
 int imparo_load_code_moe() {

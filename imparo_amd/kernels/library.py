@@ -71,6 +71,11 @@ _SIGNATURES = {
     "imparo_qk_norm_rope_store_dv": [P, P, P, F, P, I, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, P],
     "imparo_attention_dv": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, P],
     "imparo_moe_route": [P, P, P, P, I, I, I, P],
+    "imparo_moe_route_plan_tokens": [],
+    "imparo_moe_route_plan": [P, P, P, P, I, I, I, I, I, P, P, P, I, P],
+    # x, y, h, h_dtype, choice, weight, slot_of_entry, top, n_experts, n_rows_x, rows, w_post, eps_post, w_next, eps_next,
+    # out, out_dtype, n_out, width, stream
+    "imparo_post_norm_add_moe": [P, P, P, I, P, P, P, I, I, I, P, P, F, P, F, P, I, I, I, P],
     "imparo_moe_tile_rows": [I, I, I],
     "imparo_moe_max_tiles": [I, I, I],
     "imparo_moe_plan": [P, I, I, I, P, P, P, I, P],

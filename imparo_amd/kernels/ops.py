@@ -761,6 +761,25 @@ def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], choice: 
         n, r, top, _stream()), "moe_route")
 
 
+def moe_route_plan_tokens() -> int:
+    """The most tokens `moe_route_plan` takes."""
+    return int(library().imparo_moe_route_plan_tokens())
+
+
+def moe_route_plan(logits: torch.Tensor, correction: Optional[torch.Tensor], choice: torch.Tensor, weight: torch.Tensor,
+                   top: int, n_experts: int, tile_rows: int, slot_of_entry: torch.Tensor, entry_of_slot: torch.Tensor,
+                   tiles: torch.Tensor) -> None:
+    """`moe_route` and `moe_plan` in one launch, for the few tokens of a decode step."""
+    n, r = logits.shape
+    _dev(slot_of_entry, "slot_of_entry", torch.int32, (n * top,))
+    _dev(entry_of_slot, "entry_of_slot", torch.int32, (n * top,))
+    _check(library().imparo_moe_route_plan(
+        _dev(logits, "router logits", torch.float32), _dev(correction, "router correction", torch.float32, (r,)),
+        _dev(choice, "choice", torch.int32, (n, top)), _dev(weight, "choice weights", torch.float32, (n, top)),
+        n, r, top, n_experts, tile_rows, slot_of_entry.data_ptr(), entry_of_slot.data_ptr(),
+        _dev(tiles, "tiles", torch.int32), tiles.shape[0], _stream()), "moe_route_plan")
+
+
 def moe_tile_rows(n_entries: int, n_experts: int, dtype: torch.dtype) -> int:
     return int(library().imparo_moe_tile_rows(int(n_entries), int(n_experts), 0 if dtype == torch.float32 else 1))
 
@@ -813,15 +832,33 @@ def moe_combine(y: torch.Tensor, h: torch.Tensor, choice: torch.Tensor, weight: 
     return out
 
 
-def post_norm_add(x: torch.Tensor, delta: torch.Tensor, w_post: torch.Tensor, eps_post: float,
+def post_norm_add(x: torch.Tensor, delta, w_post: torch.Tensor, eps_post: float,
                   w_next: Optional[torch.Tensor] = None, eps_next: float = 0.0, out: Optional[torch.Tensor] = None,
                   rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """x += rms_norm(delta) * w_post (delta shaped like x, or [slices, *x.shape], added in order); with
-    `w_next`, out = rms_norm(x) * w_next. With `rows` only those rows are taken, into out, and x stays."""
+    `w_next`, out = rms_norm(x) * w_next. With `rows` only those rows are taken, into out, and x stays.
+    `delta` may be what a routed feed-forward left to be combined (an object with y, h, choice, weight,
+    slot_of_entry, n_experts): the launch then makes moe_combine's sum itself."""
     n_x, width = x.shape
+    n_out = n_x if rows is None else rows.shape[0]
+    if not isinstance(delta, torch.Tensor):
+        top = delta.choice.shape[1]
+        if w_next is not None and (out is None or tuple(out.shape) != (n_out, width)):
+            raise KernelArgumentError("post_norm_add: the next norm needs an output of one row per taken row")
+        if w_next is None and rows is not None:
+            raise KernelArgumentError("post_norm_add: a row selection without a next norm has no result")
+        _check(library().imparo_post_norm_add_moe(
+            _dev(x, "stream", torch.float32), _dev(delta.y, "experts' results", torch.float32),
+            _dev(delta.h, "feed-forward input", None, (n_x, width)), _code(delta.h, "feed-forward input"),
+            _dev(delta.choice, "choice", torch.int32, (n_x, top)), _dev(delta.weight, "choice weights", torch.float32, (n_x, top)),
+            _dev(delta.slot_of_entry, "slot_of_entry", torch.int32, (n_x * top,)), top, int(delta.n_experts), n_x,
+            _dev(rows, "rows", torch.int32), _dev(w_post, "post norm weight", torch.float32, (width,)), float(eps_post),
+            _dev(w_next, "next norm weight", torch.float32, (width,)), float(eps_next),
+            _dev(out, "normed") if w_next is not None else None, _code(out, "normed") if w_next is not None else 0,
+            n_out, width, _stream()), "post_norm_add")
+        return out
     n_delta = delta.shape[0] if delta.dim() == 3 else 1
     _dev(delta, "sublayer result", torch.float32, ((n_delta, n_x, width) if delta.dim() == 3 else (n_x, width)))
-    n_out = n_x if rows is None else rows.shape[0]
     if w_next is not None:
         if out is None or tuple(out.shape) != (n_out, width):
             raise KernelArgumentError("post_norm_add: the next norm needs an output of one row per taken row")

@@ -151,3 +151,17 @@ class Residual:
     # (weight, eps) of an RMS norm that the pending delta goes through before it is added (a block that
     # norms what its sublayers return); the norm that adds the delta applies it in the same launch
     post: Optional[Tuple[torch.Tensor, float]] = None
+
+
+@dataclass
+class RowsToCombine:
+    """What a routed feed-forward may leave pending on the stream instead of a finished delta: its
+    experts' rows `y` [slots, width], its input `h`, and per token the chosen experts, their weights and
+    the slots of their rows. The delta is sum_j weight[t, j] * (y[slot] or, for an expert past
+    `n_experts`, h[t]); the norm that adds it makes that sum in its own launch."""
+    y: torch.Tensor
+    h: torch.Tensor
+    choice: torch.Tensor
+    weight: torch.Tensor
+    slot_of_entry: torch.Tensor
+    n_experts: int

@@ -102,8 +102,12 @@ class SandwichBlock(PreNormBlock):
         h = self.mixer_norm.forward(ctx, res, self.mixer.in_dtype)
         res.pending, res.post = self.mixer.forward(ctx, site, owns_cache, h), self.mixer_post.as_post()
         if self.ffn is not None:
-            n = self.ffn_norm.forward(ctx, res, self.ffn.in_dtype)
-            res.pending, res.post = self.ffn.forward(ctx, n), self.ffn_post.as_post()
+            # (a buffer of its own: the feed-forward may leave this input to be read by the launch of the next
+            # norm, which writes its own result where norms usually do)
+            n = self.ffn_norm.forward(ctx, res, self.ffn.in_dtype, name="normed_ffn")
+            # a feed-forward that can leave its last sum to the norm's launch does (`forward_rows`)
+            run = getattr(self.ffn, "forward_rows", None) or self.ffn.forward
+            res.pending, res.post = run(ctx, n), self.ffn_post.as_post()
 
     def can_emit(self) -> bool:
         return False          # the step program knows the pre-norm block only

@@ -28,7 +28,7 @@ import torch
 from ..config.plan import PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
-from .base import Declared, StepContext
+from .base import Declared, RowsToCombine, StepContext
 from .linear import Linear, place_matrix, place_projection, place_vector
 from .registry import register_part
 
@@ -90,13 +90,14 @@ class RoutedExperts:
     def in_dtype(self) -> torch.dtype:
         return self.router.in_dtype
 
-    def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
+    def forward_rows(self, ctx: StepContext, n: torch.Tensor) -> RowsToCombine:
+        """Everything but the weighted sum over a token's experts: for a block whose next launch (a norm on
+        this part's result) makes that sum itself."""
         T, top, X = n.shape[0], self.top, self.experts
         ws = ctx.workspace
         z = self.router(ctx, n, torch.float32, "router_logits")
         choice = ws.get("moe_choice", (T, top), torch.int32)
         weight = ws.get("moe_weight", (T, top), torch.float32)
-        ops.moe_route(z, self.correction, choice, weight, top)
         entries = T * top
         slot_of_entry = ws.get("moe_slot_of_entry", (entries,), torch.int32)
         y = ws.get("moe_y", (entries, self.width), torch.float32)
@@ -104,12 +105,22 @@ class RoutedExperts:
             rows = ops.moe_tile_rows(entries, X, self.up.dtype)
             tiles = ws.get("moe_tiles", (ops.moe_max_tiles(entries, X, rows), 3), torch.int32)
             entry_of_slot = ws.get("moe_entry_of_slot", (entries,), torch.int32)
-            ops.moe_plan(choice, X, rows, slot_of_entry, entry_of_slot, tiles)
+            if T <= ops.moe_route_plan_tokens():      # a decode step: choice and plan in one launch
+                ops.moe_route_plan(z, self.correction, choice, weight, top, X, rows, slot_of_entry, entry_of_slot, tiles)
+            else:
+                ops.moe_route(z, self.correction, choice, weight, top)
+                ops.moe_plan(choice, X, rows, slot_of_entry, entry_of_slot, tiles)
             hidden = ws.get("moe_hidden", (entries, self.up.shape[1]), self.up.dtype, alias="mixer_in")
             ops.moe_gemm(n, self.up, hidden, tiles, rows, entry_of_slot, gather_div=top, epilogue=self.activation)
             ops.moe_gemm(hidden, self.down, y, tiles, rows)
-        out = ws.get("ffn_out", (T, self.width), torch.float32)
-        return ops.moe_combine(y, n, choice, weight, slot_of_entry, X, out)
+        else:
+            ops.moe_route(z, self.correction, choice, weight, top)
+        return RowsToCombine(y, n, choice, weight, slot_of_entry, X)
+
+    def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
+        r = self.forward_rows(ctx, n)
+        out = ctx.workspace.get("ffn_out", (n.shape[0], self.width), torch.float32)
+        return ops.moe_combine(r.y, r.h, r.choice, r.weight, r.slot_of_entry, r.n_experts, out)
 
 
 register_part("feed_forward", "routed_experts", RoutedExperts)

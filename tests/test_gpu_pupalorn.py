@@ -153,6 +153,20 @@ def test_routed_experts_part(T, E, F, X, I, top, dtype):
         got = part.forward(ctx, dev(h, part.in_dtype)).cpu()
         rel = 2e-6 if dtype == torch.float32 or part.in_dtype == torch.float32 else 6e-3    # the hidden is rounded to bfloat16
         assert float((got - ref).abs().max()) <= rel * float(ref.abs().max()), (T, E, F, X, I, top)
+    # the weighted sum left to the launch of the norm behind the part: the same bits as sum, then norm
+    from imparo_amd.kernels import ops
+    g2 = torch.Generator().manual_seed(1)
+    x, w_post, w_next = torch.randn(T, E, generator=g2), torch.rand(E, generator=g2) + 0.5, torch.rand(E, generator=g2) + 0.5
+    x1, out1 = dev(x), torch.empty(T, E, dtype=torch.float32, device=DEV)
+    ops.post_norm_add(x1, part.forward(ctx, dev(h, part.in_dtype)), dev(w_post), 1e-5, dev(w_next), 1e-6, out1)
+    x2, out2 = dev(x), torch.empty(T, E, dtype=torch.float32, device=DEV)
+    ops.post_norm_add(x2, part.forward_rows(ctx, dev(h, part.in_dtype)), dev(w_post), 1e-5, dev(w_next), 1e-6, out2)
+    assert torch.equal(x1.cpu(), x2.cpu()) and torch.equal(out1.cpu(), out2.cpu())
+    rows = i32([T - 1, 0])
+    out3 = torch.empty(2, E, dtype=torch.float32, device=DEV)
+    x3 = dev(x)
+    ops.post_norm_add(x3, part.forward_rows(ctx, dev(h, part.in_dtype)), dev(w_post), 1e-5, dev(w_next), 1e-6, out3, rows=rows)
+    assert torch.equal(x3.cpu(), x) and torch.equal(out3.cpu(), out1.cpu()[[T - 1, 0]])
 
 
 def attention_case(H, G, D, V, segments, page, dtype, window, boost=None, seed=0):
