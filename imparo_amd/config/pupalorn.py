@@ -3,7 +3,7 @@
 A Pupalorn model is a decoder whose layers are listed one by one in
 config.json (`layers`: each with a `type`, the `mixer`'s sizes and an `mlp` or
 null). Every sublayer sits between two norms, x += m * ls * post(f(pre(x))),
-with norm weights stored around zero, a layer scale `ls` per sublayer and one
+with norm weights kept as their distance from one, a layer scale `ls` per sublayer and one
 residual multiplier `m`. The mixer is grouped-query attention with per-head
 query and key norms, a rotation of part of each head whose frequencies may be
 rescaled by wavelength, and a sliding window; a layer may have no keys and

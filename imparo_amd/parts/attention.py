@@ -8,8 +8,7 @@ then the output projection
 /root/reference/crates/imparo-model/src/cpu_support.rs:361-445).
 
 Parameters beyond the sizes: `value_dim` (a head's values where they are not
-head_dim wide), `window` (a query sees itself and the window - 1 positions
-before it), `keep_window` (what the cache keeps, where a layer that reads this
+head_dim wide), `window` (a query at position i sees positions i - window + 1 .. i), `keep_window` (what the cache keeps, where a layer that reads this
 layer's cache looks further back than this layer itself; None: everything),
 `shared_kv` (the layer has no key and value projections: it is run with
 another layer's cache, `LayerCall.cache_of`, and brings queries only),

@@ -6,8 +6,8 @@ precedes a norm is fused into it (the reference's add_rms_norm,
 With `groups` > 1 the row is cut into that many equal consecutive parts and
 each is divided by its own root mean square; the weight spans the whole row.
 `tensor` names the weight outright where a checkpoint does not call it
-`<prefix>.weight`. `offset` is added to the stored weight (1 for a weight kept
-around zero). `scale_tensor` names a second vector of the row's width and
+`<prefix>.weight`. `offset` is added to the stored weight (1 where a file keeps a weight's
+distance from one). `scale_tensor` names a second vector of the row's width and
 `multiplier` a constant that the normed row is multiplied by as well (a layer
 scale and a residual multiplier on a norm that sits behind a sublayer): all
 three are folded into one float32 weight when the model is loaded.
@@ -39,7 +39,7 @@ class RmsNorm:
 
     @classmethod
     def declare(cls, spec: PartSpec) -> Declared:
-        # a weight that an offset of 1 is added to is stored around zero
+        # a weight that an offset of 1 is added to is drawn near zero
         out = {cls._tensor(spec): (TensorDecl((spec["width"],), "vector"), "bias" if spec.get("offset") else "norm")}
         if spec.get("scale_tensor"):
             out[spec["scale_tensor"]] = (TensorDecl((spec["width"],), "vector"), "norm")

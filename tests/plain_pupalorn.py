@@ -18,7 +18,7 @@ from plain_tumadra import read_safetensors, rms
 
 
 def offset_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
-    """RMS norm whose stored weight lies around zero: x / rms(x) * (1 + w)."""
+    """RMS norm whose file keeps w - 1: x / rms(x) * (1 + w)."""
     return rms(x, eps) * (1.0 + w)
 
 

@@ -1,5 +1,5 @@
 """Small Pupalorn configurations with random weights, for tests. The weights are drawn so that every
-mechanism matters: projections of unit gain, norm weights stored around zero, layer scales of order one,
+mechanism matters: projections of unit gain, norm weights kept as their distance from one, layer scales of order one,
 a router whose scores spread and a correction large enough to change some choices."""
 import json
 import math
