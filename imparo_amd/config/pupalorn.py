@@ -157,7 +157,9 @@ class PupalornConfig:
                 other = self.layers[src].mixer
                 if other.get("kv_from") is not None:
                     raise Inconsistent(f"{where}.kv_from names layer {src}, which has no keys and values of its own")
-                for key in ("heads", "kv_heads", "dim", "vdim", "rot"):
+                # the cache's shape must be the reader's own; its rotation is applied to its own queries as its
+                # own entry says (a model whose layers rotate differently has said so itself)
+                for key in ("heads", "kv_heads", "dim", "vdim"):
                     if other.get(key) != m.get(key):
                         raise Inconsistent(f"{where}: {key} differs from layer {src}'s, whose keys and values it reads")
             if layer.mlp is not None:

@@ -169,7 +169,7 @@ def test_routed_experts_part(T, E, F, X, I, top, dtype):
     assert torch.equal(x3.cpu(), x) and torch.equal(out3.cpu(), out1.cpu()[[T - 1, 0]])
 
 
-def attention_case(H, G, D, V, segments, page, dtype, window, boost=None, seed=0):
+def attention_case(H, G, D, V, segments, page, dtype, window, boost=None, seed=0, kernel="wave"):
     """q, k, v for rows given as (start, tokens) whose earlier positions are in the cache; pages in a shuffled
     order. -> (kernel output [tokens, H * V], plain output). `boost` (row, key position): that key is made to
     match the row's last query, so that it takes most of the weight if it is seen at all."""
@@ -197,7 +197,22 @@ def attention_case(H, G, D, V, segments, page, dtype, window, boost=None, seed=0
     ctx = hand_context(segments, page, n_pages, dtype, torch.device(DEV), tables=tables)
     q = dev(torch.cat(q_all), dtype)
     out = torch.empty(q.shape[0], H * V, dtype=dtype, device=DEV)
-    ops.attention(q, dev(kc, dtype), dev(vc, dtype), out, ctx.positions, ctx.row_of_token, ctx.block_tables[0], scale, window)
+    if kernel == "wave":
+        ops.attention(q, dev(kc, dtype), dev(vc, dtype), out, ctx.positions, ctx.row_of_token, ctx.block_tables[0], scale, window)
+        return out.float().cpu(), torch.cat(ref_all)
+    # the matrix-core kernels with exact weights: V transposed inside a page, single tokens and portions apart
+    assert D == V and dtype == torch.bfloat16
+    kd, vd = dev(kc, dtype), dev(vc.permute(0, 1, 3, 2), dtype)
+    if ctx.n_single_rows:
+        splits = (ctx.max_context + ops.decode_split() - 1) // ops.decode_split()
+        part_o = torch.zeros(ctx.n_single_rows * H * splits * D, device=DEV)
+        part_ml = torch.zeros(ctx.n_single_rows * H * splits * 2, device=DEV)
+        ops.attention_decode(q, kd, vd, out, part_o, part_ml, ctx.single_rows, ctx.n_single_rows, ctx.seg_start,
+                             ctx.positions, ctx.block_tables[0], scale, window, ctx.max_context, exact=True)
+    if ctx.n_portion_rows:
+        tiles = sum((n + 63) // 64 for n in ctx.host_seg_len if n > 1)
+        ops.attention_prefill(q, kd, vd, out, ctx.portion_rows, ctx.n_portion_rows, tiles, ctx.seg_start, ctx.seg_len,
+                              ctx.positions, ctx.block_tables[0], scale, window, exact=True)
     return out.float().cpu(), torch.cat(ref_all)
 
 
@@ -209,6 +224,21 @@ def test_attention_kernel_with_values_of_their_own_size(H, G, D, V, page, window
     got, ref = attention_case(H, G, D, V, [(150, 37), (299, 1), (0, 70), (63, 1), (0, 1)], page, dtype, window)
     rel = 2e-6 if dtype == torch.float32 else 1e-2
     assert float((got - ref).abs().max()) <= rel * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("D", [16, 64, 80, 128])
+@pytest.mark.parametrize("n_last", [1, 5, 70])
+@pytest.mark.parametrize("window,page", [(24, 16), (64, 64), (65, 64), (2, 32), (1, 16), (300, 64)])
+def test_a_key_at_the_windows_edge_on_the_matrix_cores(window, page, n_last, D):
+    """The same two cases through the matrix-core kernels with exact weights (decode and both prompt kernels)."""
+    L = 5 * 64 + 7
+    for key, seen in ((L - window, True), (L - window - 1, False)):
+        got, ref = attention_case(4, 2, D, D, [(L - n_last, n_last), (40, 1)], page, torch.bfloat16, window, boost=(0, key),
+                                  seed=key, kernel="mfma")
+        assert float((got - ref).abs().max()) <= 1e-2 * float(ref.abs().max()), (key, seen)
+        other, _ = attention_case(4, 2, D, D, [(L - n_last, n_last), (40, 1)], page, torch.bfloat16, window + (-1 if seen else 1),
+                                  boost=(0, key), seed=key, kernel="mfma")
+        assert float((other[n_last - 1] - ref[n_last - 1]).abs().max()) > 0.2 * float(ref[n_last - 1].abs().max()), (key, seen)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
