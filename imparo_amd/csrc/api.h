@@ -100,7 +100,7 @@ int imparo_attention_prefill_exact(const void* q, const void* k_cache, const voi
 
 // The two above for heads whose values have another size than their keys (value_dim): a token's row is
 // heads + kv_heads units of head_dim, then kv_heads units of value_dim; the value cache holds value_dim a
-// position and out is [tokens, heads * value_dim]; any head_dim up to 512. The store also takes rows of
+// position and out is [tokens, out_ld >= heads * value_dim] (the rest of a row zeros); any head_dim up to 512. The store also takes rows of
 // queries only (kv_heads 0, write_kv 0), for a layer that reads another layer's keys and values.
 int imparo_qk_norm_rope_store_dv(const float* qkv, const float* q_weight, const float* k_weight, float eps,
                                  const float* inv_freq, int n_freq, int interleaved,
@@ -112,7 +112,7 @@ int imparo_qk_norm_rope_store_dv(const float* qkv, const float* q_weight, const 
 int imparo_attention_dv(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
                         const int32_t* positions, const int32_t* row_of_token,
                         const int32_t* block_table, int table_stride, int page_size,
-                        int n_tokens, int heads, int kv_heads, int head_dim, int value_dim, int n_pages,
+                        int n_tokens, int heads, int kv_heads, int head_dim, int value_dim, int out_ld, int n_pages,
                         float scale, int window, int v_transposed, imparo_stream stream);
 
 // Matrix-core attention, bfloat16, V cache transposed, page_size a power of two

@@ -59,7 +59,7 @@ __global__ void k_attention_wave(const T* __restrict__ q, const T* __restrict__ 
                                  T* __restrict__ out, const int32_t* __restrict__ positions,
                                  const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ block_table,
                                  int table_stride, int page_size, int n_tokens, int heads, int kv_heads, int head_dim,
-                                 int value_dim, int n_pages, float scale, int window, int v_transposed) {
+                                 int value_dim, int out_ld, int n_pages, float scale, int window, int v_transposed) {
     __shared__ float q_rows[ATT_WAVES][ATT_MAX_HEAD_DIM];
     __shared__ float probs[ATT_WAVES][WAVE];
     __shared__ long long v_off[ATT_WAVES][WAVE];
@@ -126,12 +126,15 @@ __global__ void k_attention_wave(const T* __restrict__ q, const T* __restrict__ 
         wave_lds_sync();
     }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    T* dst = out + ((size_t)t * heads + h) * value_dim;
+    T* dst = out + (size_t)t * out_ld + (size_t)h * value_dim;
 #pragma unroll
     for (int j = 0; j < DPL; ++j) {
         const int d = lane + j * WAVE;
         if (d < value_dim) store_f32<T>(dst, d, acc[j] * inv);
     }
+    // a row wider than its heads (filled up for a product that walks it in steps of 8) ends in zeros
+    if (h == heads - 1)
+        for (int d = value_dim + lane; d < out_ld - h * value_dim; d += WAVE) store_f32<T>(dst, d, 0.f);
 }
 
 static int check_attention_args(const void* q, const void* k_cache, const void* v_cache, void* out,
@@ -146,16 +149,17 @@ static int check_attention_args(const void* q, const void* k_cache, const void* 
 }
 
 // Keys of head_dim and values of value_dim a head: q [tokens, heads, head_dim], the value cache
-// [pages, kv_heads, page, value_dim] (or transposed inside the page), out [tokens, heads * value_dim].
+// [pages, kv_heads, page, value_dim] (or transposed inside the page), out [tokens, out_ld] with out_ld >=
+// heads * value_dim; what lies beyond the heads in a row is written as zeros.
 extern "C" int imparo_attention_dv(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
                                 const int32_t* positions, const int32_t* row_of_token,
                                 const int32_t* block_table, int table_stride, int page_size,
-                                int n_tokens, int heads, int kv_heads, int head_dim, int value_dim, int n_pages,
-                                float scale, int window, int v_transposed, imparo_stream stream) {
+                                int n_tokens, int heads, int kv_heads, int head_dim, int value_dim, int out_ld,
+                                int n_pages, float scale, int window, int v_transposed, imparo_stream stream) {
     const int bad = check_attention_args(q, k_cache, v_cache, out, positions, row_of_token, block_table, table_stride,
                                          page_size, n_tokens, heads, kv_heads, head_dim, n_pages, window);
     if (bad) return bad;
-    if (value_dim <= 0 || value_dim > ATT_MAX_HEAD_DIM) return IMPARO_BAD_ARGUMENT;
+    if (value_dim <= 0 || value_dim > ATT_MAX_HEAD_DIM || out_ld < heads * value_dim) return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
     const long long total = (long long)n_tokens * heads;
     const unsigned blocks = (unsigned)((total + ATT_WAVES - 1) / ATT_WAVES);
@@ -163,11 +167,11 @@ extern "C" int imparo_attention_dv(const void* q, const void* k_cache, const voi
     if (dtype == IMPARO_F32)
         k_attention_wave<float><<<blocks, ATT_WAVES * WAVE, 0, s>>>(
             (const float*)q, (const float*)k_cache, (const float*)v_cache, (float*)out, positions, row_of_token,
-            block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, value_dim, n_pages, scale, window, v_transposed);
+            block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, value_dim, out_ld, n_pages, scale, window, v_transposed);
     else if (dtype == IMPARO_BF16)
         k_attention_wave<bf16_t><<<blocks, ATT_WAVES * WAVE, 0, s>>>(
             (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, positions, row_of_token,
-            block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, value_dim, n_pages, scale, window,
+            block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, value_dim, out_ld, n_pages, scale, window,
             v_transposed);
     else
         return IMPARO_BAD_ARGUMENT;
@@ -181,8 +185,8 @@ extern "C" int imparo_attention(const void* q, const void* k_cache, const void* 
                                 float scale, int window, int v_transposed, imparo_stream stream) {
     if (head_dim % 16 != 0) return IMPARO_BAD_ARGUMENT;
     return imparo_attention_dv(q, k_cache, v_cache, out, dtype, positions, row_of_token, block_table, table_stride,
-                               page_size, n_tokens, heads, kv_heads, head_dim, head_dim, n_pages, scale, window,
-                               v_transposed, stream);
+                               page_size, n_tokens, heads, kv_heads, head_dim, head_dim, heads * head_dim, n_pages, scale,
+                               window, v_transposed, stream);
 }
 
 // Asks the runtime about one kernel of this file, which makes it load the file's code onto the

@@ -69,7 +69,7 @@ _SIGNATURES = {
     "imparo_diff_attention_tiles": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, I, F, F, F, I, P],
     "imparo_embed_gather_scaled": [P, I, P, P, I, I, I, F, P],
     "imparo_qk_norm_rope_store_dv": [P, P, P, F, P, I, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, P],
-    "imparo_attention_dv": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, P],
+    "imparo_attention_dv": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, I, I, P],
     "imparo_moe_route": [P, P, P, P, I, I, I, P],
     "imparo_moe_route_plan_tokens": [],
     "imparo_moe_route_plan": [P, P, P, P, I, I, I, I, I, P, P, P, I, P],

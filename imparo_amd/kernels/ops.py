@@ -222,7 +222,8 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out
               positions: torch.Tensor, row_of_token: torch.Tensor, block_table: torch.Tensor,
               scale: float, window: Optional[int], v_transposed: bool = False) -> torch.Tensor:
     """The general kernel: any page size, head sizes up to 512 (values of a size of their own
-    are read off the value cache's shape), float32 or bfloat16; one wave per (token, head)."""
+    are read off the value cache's shape), float32 or bfloat16; one wave per (token, head). `out`
+    may be wider than heads x value size: the rest of a row is written as zeros."""
     n, heads, head_dim = q.shape
     n_pages, kv_heads, page_size, hd = k_cache.shape
     value_dim = v_cache.shape[2] if v_transposed else v_cache.shape[3]
@@ -230,15 +231,17 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out
         raise KernelArgumentError(f"attention: q has head size {head_dim}, the cache {hd}")
     if heads % kv_heads != 0:
         raise KernelArgumentError(f"attention: {heads} heads cannot share {kv_heads} kv heads evenly")
+    if out.dim() != 2 or out.shape[0] != n or out.shape[1] < heads * value_dim:
+        raise KernelArgumentError(f"attention: out is {list(out.shape)}; [{n}, at least {heads * value_dim}] is needed")
     _check(library().imparo_attention_dv(
         _dev(q, "q"), _dev(k_cache, "k cache", q.dtype),
         _dev(v_cache, "v cache", q.dtype, (n_pages, kv_heads, value_dim, page_size) if v_transposed
              else (n_pages, kv_heads, page_size, value_dim)),
-        _dev(out, "attention out", q.dtype, (n, heads * value_dim)), _code(q, "q"),
+        _dev(out, "attention out", q.dtype), _code(q, "q"),
         _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
         _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size,
-        n, heads, kv_heads, head_dim, value_dim, n_pages, float(scale), int(window or 0), int(v_transposed),
-        _stream()), "attention")
+        n, heads, kv_heads, head_dim, value_dim, out.shape[1], n_pages, float(scale), int(window or 0),
+        int(v_transposed), _stream()), "attention")
     return out
 
 

@@ -83,10 +83,14 @@ class Attention:
             ws = [w.to(torch.float32) for w in ws]
         # one projection for q | k | v: the same dot products, one launch
         self.qkv = Linear(place_projection(torch.cat(ws, dim=0), engine_dtype, device))
-        self.out = Linear(place_projection(tensors[n["o"] + sfx], engine_dtype, device))
-        if engine_dtype != torch.float32 and self.out.in_dtype == torch.float32:
-            raise ValueError(f"heads x value size = {self.heads * self.value_dim} must be a multiple of 8 under bfloat16 "
-                             f"(the attention kernels write their result in the cache's dtype)")
+        out = tensors[n["o"] + sfx]
+        # The attention kernels write their result in the cache's dtype and the bfloat16 products walk K in steps
+        # of 8: where heads x value size is no multiple of 8 the output projection gets columns of zero weight and
+        # the attention rows end in as many zeros.
+        self.out_fill = (-self.heads * self.value_dim) % 8 if engine_dtype != torch.float32 and out.dtype != torch.float32 else 0
+        if self.out_fill:
+            out = torch.cat([out, out.new_zeros(out.shape[0], self.out_fill)], dim=1)
+        self.out = Linear(place_matrix(out, engine_dtype, device))
         norm = spec.get("qk_norm")
         if norm is not None:
             # the kernels that norm a head know one norm: RMS with a weight per dimension, no offset
@@ -161,7 +165,7 @@ class Attention:
                                q, k_cache if owns_cache else None, v_cache if owns_cache else None,
                                self.heads, 0 if self.shared_kv else self.kv_heads, self.head_dim, v_transposed=vt,
                                interleaved=interleaved, value_dim=Dv)
-        o = ctx.workspace.get("attn_out", (T, self.heads * Dv), ctx.dtype, alias="mixer_mid")
+        o = ctx.workspace.get("attn_out", (T, self.heads * Dv + self.out_fill), ctx.dtype, alias="mixer_mid")
         if vt and ctx.single_rows is not None:
             # matrix-core kernels: single tokens split over their keys, portions tiled over their queries
             if ctx.n_single_rows:
@@ -194,7 +198,8 @@ class Attention:
 
     def can_emit(self) -> bool:
         # the step program's attention has one head size, keys and values of its own, and the matrix-core kernels
-        return self.value_dim == self.head_dim and not self.shared_kv and not self.exact_weights
+        return (self.value_dim == self.head_dim and not self.shared_kv and not self.exact_weights
+                and not self.out_fill)
 
     def emit(self, program, site: int, owns_cache: bool) -> None:
         """Appends `forward` to a native step program."""

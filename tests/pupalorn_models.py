@@ -60,6 +60,16 @@ CONFIG_C = dict(
         layer(attention(2, 1, 12, 20, window=70, rot=(4, 50.0), kv_from=0), moe(12, 2, 2, 2)),
     ])
 
+# E: heads x value size no multiple of 8 under a width that is one (the attention rows end in zeros, the output
+# projection in columns of zero weight)
+CONFIG_E = dict(
+    architecture="Pupalorn", vocab=90, width=48, norm=dict(eps=1e-5), residual_mult=0.4,
+    layers=[
+        layer(attention(3, 1, 16, 20, window=11, rot=(8, 100.0)), moe(16, 2, 1, 2)),
+        layer(attention(3, 3, 8, 4, rot=(8, 100.0)), None),
+        layer(attention(3, 1, 16, 20, window=30, rot=(8, 100.0), kv_from=0), moe(8, 3, 0, 1)),
+    ])
+
 # D: heads of 64 rotated in half, sixteen experts of which four are used, a long window
 CONFIG_D = dict(
     architecture="Pupalorn", vocab=500, width=128, norm=dict(eps=1e-5), residual_mult=0.7, embedding=dict(scale=2.0),
@@ -69,7 +79,7 @@ CONFIG_D = dict(
         layer(attention(2, 1, 128, 128, rot=(128, 10000.0), scaling=(8.0, 1.0, 4.0, 256)), moe(32, 6, 0, 2)),
     ])
 
-CONFIGS = {"A": (CONFIG_A, 21), "B": (CONFIG_B, 22), "C": (CONFIG_C, 23), "D": (CONFIG_D, 24)}
+CONFIGS = {"A": (CONFIG_A, 21), "B": (CONFIG_B, 22), "C": (CONFIG_C, 23), "D": (CONFIG_D, 24), "E": (CONFIG_E, 25)}
 
 
 def random_weights(config, seed, gain=1.0):

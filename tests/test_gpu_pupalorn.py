@@ -344,7 +344,7 @@ def test_head_norm_rotation_and_cache_write(H, G, D, V, rot, n, dtype):
 
 # ------------------------------------------------------------------ the model
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_whole_prompt_and_stepwise(dirs, plains, name, dtype):
     """A prompt whole; then most of it whole and its last 50 tokens one by one (captured steps)."""
     from imparo_amd.engine import StepEntry
@@ -365,7 +365,7 @@ def test_whole_prompt_and_stepwise(dirs, plains, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,page", [("A", 16), ("B", 8), ("C", 16), ("D", 64)])
+@pytest.mark.parametrize("name,page", [("A", 16), ("B", 8), ("C", 16), ("D", 64), ("E", 32)])
 def test_portions_of_changing_size(dirs, plains, name, page, dtype):
     """Portions down to two tokens, cut inside pages and windows, also without captured steps."""
     tokens = prompt_tokens(vocab(name), 160, 8)

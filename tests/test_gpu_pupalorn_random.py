@@ -37,9 +37,7 @@ def draw_config(seed):
             kv = rng.choice([1, 2, 3, 4])
             heads = kv * rng.choice([1, 1, 2, 3])
             dim = rng.choice([8, 16, 32, 64, 128]) if rng.random() < 0.8 else rng.choice([24, 40, 80])
-            vdim = dim if rng.random() < 0.5 else rng.choice([8, 16, 32, 64])
-            while (heads * vdim) % 8:
-                vdim += 8 - vdim % 8
+            vdim = dim if rng.random() < 0.5 else rng.choice([4, 8, 12, 16, 20, 32, 64])
             rot = None
             if rng.random() < 0.85:
                 dims = rng.choice([dim, dim // 2, dim // 4 * 2]) or 2
