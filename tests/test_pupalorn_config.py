@@ -78,3 +78,26 @@ def test_frequency_scaling_has_three_bands(dims, base, scaling):
     kept, divided = np.isclose(got, raw, rtol=1e-12), np.isclose(got, raw / scaling[0], rtol=1e-12)
     assert kept.any() and divided.any() and (~kept & ~divided).any(), "a band is not met by this case"
     assert np.all(np.diff(got) < 0)
+
+
+def test_random_weights_mode_writes_a_loadable_model(tmp_path):
+    """The seeded random-weights mode writes what the plan declares, and the by-name loader takes it back;
+    a file with a tensor that a layer on borrowed keys must not have is refused by name."""
+    from imparo_amd import WeightsError, write_random_model
+    from imparo_amd.weights import load_weights
+    from imparo_amd.weights.safetensors_io import save_file
+    cfg = CONFIGS["A"][0]
+    d = write_random_model(cfg, 5, str(tmp_path / "m"))
+    _, plan = plan_from_config(cfg)
+    declared = {k: decl for k, (decl, _) in declared_tensors(plan).items()}
+    tensors = load_weights(d, declared)
+    tensors.pop("__file__").close()
+    assert set(tensors) == set(declared)
+    assert float(tensors["l0.norm1"].float().abs().max()) < 0.2        # kept as the distance from one
+    assert abs(float(tensors["l0.ls1"].float().mean()) - 1.0) < 0.1
+    extra = dict(tensors)
+    extra["l2.mix.k"] = tensors["l0.mix.k"].clone()
+    save_file({k: v.contiguous() for k, v in extra.items()}, str(tmp_path / "m" / "model.safetensors"))
+    with pytest.raises(WeightsError) as e:
+        load_weights(d, declared)
+    assert e.value.unexpected == ["l2.mix.k"]
