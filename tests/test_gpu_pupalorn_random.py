@@ -61,10 +61,10 @@ def draw_config(seed):
             experts, identity = rng.choice([1, 2, 3, 8, 12]), rng.choice([0, 0, 1, 4])
             mlp = moe(rng.choice([8, 20, 32, 64]), experts, identity, rng.randint(1, min(4, experts + identity)))
         layers.append(layer(mixer, mlp))
-    cfg = dict(architecture="Pupalorn", vocab=rng.choice([50, 97, 300, 448]), width=width,
+    cfg = dict(architecture="Pupalorn", vocab=rng.choice([50, 97, 300, 500]), width=width,
                norm=dict(eps=rng.choice([1e-6, 1e-5, 1e-3])), layers=layers)
     if rng.random() < 0.7:
-        cfg["residual_mult"] = rng.choice([0.3, 0.5, 1.5])
+        cfg["residual_mult"] = rng.choice([0.25, 0.5, 1.5])
     if rng.random() < 0.7:
         cfg["embedding"] = dict(scale=rng.choice([0.5, 1.0, 3.0]))
     return cfg
